@@ -1,0 +1,230 @@
+"""The oracle's CpuBackend ops and permutation against the reference's own golden tests
+(crates/ferrite-kernel/tests/golden.rs, gpu_smoke.rs:139-155, dsv41/chain_dev.rs:25042-25090,
+dsv41/ops.rs:1079-1105) plus closed forms and brute force."""
+import itertools
+import math
+
+import numpy as np
+import pytest
+
+
+def sigmoid32(v):
+    v = np.float32(v)
+    return np.float32(1.0) / (np.float32(1.0) + np.float32(math.exp(-float(v))))
+
+
+def test_matmul_matches_manual(oracle):  # golden.rs:14-27
+    x = np.array([[1, 2], [3, 4]], np.float32)
+    w = np.array([[5, 6], [7, 8]], np.float32)
+    assert oracle.matmul(x, w).tolist() == [[17, 23], [39, 53]]
+    assert oracle.matmul(x, w, np.array([0.5, -0.5], np.float32)).tolist() == [[17.5, 22.5], [39.5, 52.5]]
+    with pytest.raises(oracle.OracleError):
+        oracle.matmul(x, np.zeros((2, 3), np.float32))
+
+
+def test_matmul_is_sequential_f32_chain(oracle):
+    """Bit-for-bit equal to s=0; s = fl(s + fl(x*w)) in index order; the 8-row interleave in the
+    oracle must not change any chain (rows 0..18 exercise both the blocked and the tail path)."""
+    rng = np.random.default_rng(0)
+    x = rng.normal(0, 1, (3, 301)).astype(np.float32)
+    w = rng.normal(0, 1, (19, 301)).astype(np.float32)
+    got = oracle.matmul(x, w)
+    for i in range(3):
+        for j in range(19):
+            s = np.float32(0)
+            for l in range(301):
+                s = np.float32(s + np.float32(x[i, l] * w[j, l]))
+            assert got[i, j] == s
+    # and it is NOT the fused-multiply-add chain on at least one element (contraction is off)
+    diff = 0
+    for j in range(19):
+        s = 0.0
+        sf = np.float32(0)
+        for l in range(301):
+            sf = np.float32(float(sf) + float(x[0, l]) * float(w[j, l]))  # fma-like: one rounding
+        diff += int(sf != got[0, j])
+    assert diff > 0
+
+
+def test_swiglu_clamps(oracle):  # golden.rs:44-55
+    out = oracle.swiglu_limited(np.array([[2., 20., 3., 1.]], np.float32), 10.0)
+    silu2 = 2.0 / (1.0 + math.exp(-2.0))
+    assert abs(out[0, 0] - silu2 * 3.0) < 1e-6
+    assert abs(out[0, 1] - 10.0 / (1.0 + math.exp(-10.0))) < 1e-6
+
+
+def test_swiglu_up_clamps_both_sides(oracle):  # dsv41 ops.rs:1100-1105: silu(10) * -10
+    out = oracle.swiglu_limited(np.array([[100., -100.]], np.float32), 10.0)
+    assert abs(out[0, 0] - (10.0 / (1.0 + math.exp(-10.0))) * -10.0) < 1e-4
+    out = oracle.swiglu_limited(np.array([[-100., 100.]], np.float32), 10.0)   # gate is not clamped below
+    assert abs(out[0, 0] - (-100.0 / (1.0 + math.exp(100.0))) * 10.0) < 1e-30
+
+
+def test_moe_route_noaux_tc(oracle):  # golden.rs:189-210
+    probs, ids = oracle.moe_route(np.array([[1.0, 2.0, 0.5]]), np.array([0.0, 0.0, 0.5]), 2, 1.0)
+    assert ids.tolist() == [[2.0, 1.0]]
+    s1, s2 = sigmoid32(2.0), sigmoid32(0.5)
+    assert abs(probs[0, 0] - s2 / (s1 + s2)) < 1e-5
+    assert abs(probs[0, 1] - s1 / (s1 + s2)) < 1e-5
+
+
+def test_moe_route_bias_selects_but_does_not_scale(oracle):  # dsv41 ops.rs:1079-1087
+    probs, ids = oracle.moe_route(np.array([[1.0, 1.0]]), np.array([0.0, 10.0]), 1, 1.0)
+    assert ids[0, 0] == 1.0
+    s = float(sigmoid32(1.0))
+    assert abs(probs[0, 0] - s / (s + np.finfo(np.float32).eps)) < 1e-6
+
+
+def ramp_fixture():
+    n, e, topk = 2, 288, 8
+    logits = (np.arange(n * e, dtype=np.float32) * np.float32(0.017) - np.float32(2.0)).reshape(n, e)
+    bias = ((np.arange(e) % 11).astype(np.float32) * np.float32(0.01))
+    return logits, bias, topk
+
+
+def test_moe_route_ramp_fixture_closed_form(oracle):  # gpu_smoke.rs:139-155 inputs
+    logits, bias, topk = ramp_fixture()
+    probs, ids = oracle.moe_route(logits, bias, topk, 2.5)
+    for r in range(2):
+        sig = 1.0 / (1.0 + np.exp(-logits[r].astype(np.float64)))
+        choice = sig + bias
+        order = sorted(range(288), key=lambda j: (-choice[j], j))[:topk]
+        assert ids[r].astype(int).tolist() == order
+        want = sig[order] / sig[order].sum() * 2.5
+        assert np.allclose(probs[r], want, atol=1e-5)
+        assert len(set(order)) == topk
+        assert abs(probs[r].sum() - 2.5) < 1e-4
+
+
+def test_moe_route_ties_go_to_lower_index_and_order_is_by_choice(oracle):  # cpu.rs:560
+    logits = np.zeros((1, 8), np.float32)
+    probs, ids = oracle.moe_route(logits, np.zeros(8, np.float32), 3, 1.0)
+    assert ids.tolist() == [[0.0, 1.0, 2.0]]
+    bias = np.array([0, 0.25, 0, 0.25, 0.5, 0, 0, 0], np.float32)
+    _, ids = oracle.moe_route(logits, bias, 4, 1.0)
+    assert ids.tolist() == [[4.0, 1.0, 3.0, 0.0]]
+
+
+def test_moe_route_brute_force_small(oracle):
+    rng = np.random.default_rng(2)
+    for _ in range(50):
+        e, k = int(rng.integers(2, 9)), 0
+        k = int(rng.integers(1, e + 1))
+        logits = rng.normal(0, 2, (1, e)).astype(np.float32)
+        bias = rng.normal(0, 0.3, e).astype(np.float32)
+        probs, ids = oracle.moe_route(logits, bias, k, 1.7)
+        sig = np.array([sigmoid32(v) for v in logits[0]], np.float32)
+        choice = (sig + bias).astype(np.float32)
+        # the k chosen experts maximise the sum of choice scores over all k-subsets
+        best = max(itertools.combinations(range(e), k), key=lambda c: sum(float(choice[j]) for j in c))
+        assert sorted(ids[0].astype(int).tolist()) == sorted(best)
+        ch = [float(choice[int(j)]) for j in ids[0]]
+        assert ch == sorted(ch, reverse=True)
+        s = np.float32(0)
+        for j in ids[0].astype(int):
+            s = np.float32(s + sig[j])
+        want = [np.float32(np.float32(sig[j] / np.float32(s + np.finfo(np.float32).eps)) * np.float32(1.7))
+                for j in ids[0].astype(int)]
+        assert probs[0].tolist() == want
+
+
+def test_moe_route_nan_is_an_error(oracle):  # the reference's partial_cmp().unwrap() panics
+    with pytest.raises(oracle.OracleError):
+        oracle.moe_route(np.array([[np.nan, 1.0]]), np.zeros(2), 1, 1.0)
+    with pytest.raises(oracle.OracleError):
+        oracle.moe_route(np.zeros((1, 4)), np.zeros(3), 1, 1.0)
+
+
+# ---- group-limited routing: no reference counterpart (parity unpinned); pinned by reduction + brute force
+def test_grouped_reduces_to_plain_router(oracle):
+    rng = np.random.default_rng(4)
+    logits = rng.normal(0, 1.5, (16, 32)).astype(np.float32)
+    bias = rng.normal(0, 0.05, 32).astype(np.float32)
+    p0, i0 = oracle.moe_route(logits, bias, 6, 2.5)
+    for ng, tg in [(1, 1), (4, 4), (8, 8), (32, 32)]:
+        p, i = oracle.moe_route(logits, bias, 6, 2.5, ng, tg)
+        assert np.array_equal(i, i0) and np.array_equal(p, p0)
+
+
+def test_grouped_brute_force_c0_shape(oracle):
+    """E=16, 4 groups keep 2, top-4: enumerate all C(4,2) group subsets."""
+    rng = np.random.default_rng(6)
+    logits = rng.normal(0, 1.5, (64, 16)).astype(np.float32)
+    bias = rng.normal(0, 0.05, 16).astype(np.float32)
+    probs, ids = oracle.moe_route(logits, bias, 4, 2.5, 4, 2)
+    for r in range(64):
+        sig = np.array([sigmoid32(v) for v in logits[r]], np.float32)
+        choice = (sig + bias).astype(np.float32)
+        gscore = []
+        for g in range(4):
+            top2 = sorted(choice[g * 4:(g + 1) * 4].tolist(), reverse=True)[:2]
+            gscore.append(float(np.float32(np.float32(top2[0]) + np.float32(top2[1]))))
+        best = max(itertools.combinations(range(4), 2), key=lambda c: (gscore[c[0]] + gscore[c[1]]))
+        kept = sorted(range(4), key=lambda g: (-gscore[g], g))[:2]
+        assert sorted(kept) == sorted(best)
+        cand = [j for j in range(16) if j // 4 in kept]
+        want = sorted(cand, key=lambda j: (-float(choice[j]), j))[:4]
+        assert ids[r].astype(int).tolist() == want
+        assert all(int(j) // 4 in kept for j in ids[r])
+
+
+def test_grouped_rejects_bad_shapes(oracle):
+    z = np.zeros((1, 16), np.float32)
+    with pytest.raises(oracle.OracleError):
+        oracle.moe_route(z, np.zeros(16), 4, 1.0, 3, 2)      # E % n_group
+    with pytest.raises(oracle.OracleError):
+        oracle.moe_route(z, np.zeros(16), 9, 1.0, 4, 2)      # topk > kept experts
+
+
+# ---- permutation
+def test_moe_align_host_groups_stably_and_zero_fills(oracle):  # chain_dev.rs:25042-25061
+    BM, CAP = 8, 16
+    order, counts, eid, nseg = oracle.moe_align_host([5, 1, 5, 1, 5, 2, 9, 1, 9], 3, CAP, BM)
+    assert nseg == 4
+    assert eid[:4].tolist() == [1, 2, 5, 9]
+    assert counts[:4].tolist() == [3, 1, 3, 2]
+    assert order[0:3].tolist() == [1, 3, 7]
+    assert order[BM:BM + 1].tolist() == [5]
+    assert order[2 * BM:2 * BM + 3].tolist() == [0, 2, 4]
+    assert order[3 * BM:3 * BM + 2].tolist() == [6, 8]
+    assert order[3] == -1 and np.all(order[nseg * BM:] == -1) and np.all(counts[nseg:] == 0)
+
+
+def test_moe_align_host_declines_out_of_contract(oracle):  # chain_dev.rs:25077-25090
+    assert oracle.moe_align_host([], 6, 16, 8) is None
+    assert oracle.moe_align_host([0, 1, 2], 0, 16, 8) is None
+    assert oracle.moe_align_host([0, -1, 2], 3, 16, 8) is None
+    assert oracle.moe_align_host(list(range(17)), 1, 16, 8) is None
+    assert oracle.moe_align_host([7] * 9, 1, 16, 8) is None
+
+
+def test_moe_permute_reference_vector(oracle):  # same routing table, dsv41_route.cu:194-225 tables
+    ids = np.array([[5, 1, 5], [1, 5, 2], [9, 1, 9]], np.int32)
+    t = oracle.moe_permute(ids, 12)
+    assert t["counts"].tolist() == [0, 3, 1, 0, 0, 3, 0, 0, 0, 2, 0, 0]
+    assert t["gather_src"].tolist() == [1, 3, 7, 5, 0, 2, 4, 6, 8]
+    assert t["active"][:t["n_active"]].tolist() == [1, 2, 5, 9] and t["n_active"] == 4
+    assert t["starts"].tolist() == [0, 0, 3, 4, 4, 4, 7, 7, 7, 7, 9, 9, 9]
+    assert t["perm_map"].tolist() == [4, 0, 5, 1, 6, 3, 7, 2, 8]
+
+
+def test_moe_permute_is_stable_sort_and_invariants(oracle):
+    rng = np.random.default_rng(8)
+    for n, k, e in [(1, 1, 1), (7, 3, 5), (64, 8, 128), (300, 8, 256)]:
+        ids = np.stack([rng.permutation(e)[:k] if k <= e else rng.integers(0, e, k) for _ in range(n)]).astype(np.int32)
+        t = oracle.moe_permute(ids, e)
+        flat = ids.ravel()
+        want = np.argsort(flat, kind="stable")
+        assert np.array_equal(t["gather_src"], want)
+        assert np.array_equal(t["perm_map"][t["gather_src"]], np.arange(n * k))
+        assert np.array_equal(t["counts"], np.bincount(flat, minlength=e))
+        assert np.array_equal(t["starts"], np.concatenate([[0], np.cumsum(t["counts"])]))
+        assert t["counts"].sum() == n * k
+
+
+def test_moe_permute_out_of_range_ids_drop_out(oracle):  # dsv41_route.cu:253-261,300-303
+    ids = np.array([[0, 7], [-1, 0]], np.int32)
+    t = oracle.moe_permute(ids, 4)
+    assert t["perm_map"].tolist() == [0, -1, -1, 1]
+    assert t["gather_src"].tolist() == [0, 3, -1, -1]
+    assert t["starts"][-1] == 2
