@@ -1,0 +1,57 @@
+"""Builds libferrite_hip.so for gfx950 with hipcc (in-tree, next to the sources).
+
+`python -m ferrite_amd.build` or ferrite_amd.build.build().  The build id baked into the library is a hash of
+every source that goes into it (the same-source gate of the reference, crates/ferrite-kernel/build.rs:1-216).
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+SO_PATH = os.path.join(HERE, "libferrite_hip.so")
+SOURCES = ["layer.hip", "route.hip", "formats.hip", "experts_f32.hip", "experts_mfma.hip"]
+HEADERS = ["internal.hpp", "numerics.hpp"]
+
+
+def source_hash() -> str:
+    h = hashlib.sha256()
+    for name in SOURCES + HEADERS:
+        with open(os.path.join(CSRC, name), "rb") as f:
+            h.update(name.encode())
+            h.update(f.read())
+    with open(os.path.join(INCLUDE, "ferrite_hip.h"), "rb") as f:
+        h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every HIP source into libferrite_hip.so (always recompiles)."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    build_id = "ferrite-hip-" + source_hash()
+    cmd = [hipcc, "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           # a*b+c must stay two rounded operations: routing has to reproduce the reference's f32 chains bit
+           # for bit (HIP's __fmul_rn/__fadd_rn are plain operators and would otherwise be fused); fmaf() where
+           # a fused multiply-add is wanted is written explicitly
+           "-ffp-contract=off",
+           "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
+           f'-DFERRITE_BUILD_ID="{build_id}"', "-I", INCLUDE, "-o", SO_PATH]
+    cmd += [os.path.join(CSRC, s) for s in SOURCES]
+    if verbose:
+        print(" ".join(cmd))
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("hipcc failed")
+    if verbose and res.stderr:
+        sys.stderr.write(res.stderr)
+    return SO_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

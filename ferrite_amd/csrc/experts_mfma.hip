@@ -1,0 +1,493 @@
+// Expert GEMMs on the CDNA4 block-scaled MFMA (v_mfma_scale_f32_16x16x128_f8f6f4): e2m1 weights with their
+// e8m0-per-32 scales go from HBM straight into the matrix core, activations are e4m3 with e8m0-per-32 scales.
+//
+// Orientation: weights are the A operand (16 weight rows x 128 k per instruction), tokens are the B operand
+// (16 token columns), so a unit of up to 16 tokens that share an expert streams every byte of that expert's
+// weights exactly once.  Operand layouts of the instruction (measured on gfx950):
+//   A (e2m1, 4 VGPRs): lane l holds row l%16, k = 32*(l/16) + [0,32), low nibble = lower k
+//   B (e4m3, 8 VGPRs): lane l holds column l%16; VGPR 0-3 = k 16*(l/16) + [0,16), VGPR 4-7 = k 64 + 16*(l/16) + [0,16)
+//   scale operands   : lane l, byte op_sel = e8m0 of row/column l%16 for the k block 32*(l/16) + [0,32)
+//   D (f32, 4 VGPRs) : lane l, VGPR v = element (row 4*(l/16) + v, column l%16)
+//
+// The packed weight buffer stores, per work item (32 gate rows + the same 32 up rows, or 64 down rows), the
+// code tiles in exactly the order a wave consumes them: [item][k step][tile 0..3][lane][16 B], so a wave
+// reads one contiguous 4 KiB per k step with 128-bit loads; scales are [item][4 k steps][lane][tile][4 B].
+#include "internal.hpp"
+#include "numerics.hpp"
+
+namespace fe {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned int u4v __attribute__((ext_vector_type(4)));  // 128-bit vector usable with nontemporal loads
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+PackedLayout packed_layout(const ferrite_moe_shape& s) {
+    PackedLayout L{};
+    const size_t H = s.hidden, I = s.inter, Is = s.shared_inter, E = s.n_experts;
+    auto kt4 = [](size_t K) { return (K / 128 + 3) / 4; };
+    L.gu_codes_per_expert = I * H;                               // (I/32 items) * (H/128) * 4096
+    L.gu_scales_per_expert = (I / 32) * kt4(H) * 1024;
+    L.dn_codes_per_expert = H * I / 2;                           // (H/64 items) * (I/128) * 4096
+    L.dn_scales_per_expert = (H / 64) * kt4(I) * 1024;
+    size_t off = 0;
+    L.gu_codes = off;  off = align_up(off + E * L.gu_codes_per_expert, 256);
+    L.gu_scales = off; off = align_up(off + E * L.gu_scales_per_expert, 256);
+    L.dn_codes = off;  off = align_up(off + E * L.dn_codes_per_expert, 256);
+    L.dn_scales = off; off = align_up(off + E * L.dn_scales_per_expert, 256);
+    L.sh_gu_codes = off;  off = align_up(off + Is * H, 256);
+    L.sh_gu_scales = off; off = align_up(off + (Is / 32) * kt4(H) * 1024, 256);
+    L.sh_dn_codes = off;  off = align_up(off + H * Is / 2, 256);
+    L.sh_dn_scales = off; off = align_up(off + (H / 64) * kt4(Is) * 1024, 256);
+    L.total = off;
+    return L;
+}
+
+// ---- packing: a pure permutation of bytes --------------------------------------------------------
+// An item covers `rpi` rows of each of `nmat` source matrices (gate_up: rpi 32, nmat 2; down: rpi 64, nmat 1);
+// its 4 tiles are 16-row slices: tile -> (matrix tile / (4/nmat), rows (tile % (4/nmat))*16 ..).
+struct PackSrc {
+    const uint8_t* codes[2];
+    const uint8_t* scales[2];
+    int rows, K;       // rows per matrix, columns
+    int nmat, rpi;
+};
+
+__global__ __launch_bounds__(256) void pack_codes_kernel(PackSrc s, int n_experts, uint4* __restrict__ dst) {
+    const int KT = s.K / 128;
+    const size_t items = s.rows / s.rpi;
+    const size_t per_expert = items * KT * 4 * 64;  // uint4 per expert
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= per_expert * n_experts) return;
+    size_t e = idx / per_expert, r = idx % per_expert;
+    int lane = r & 63;
+    int tile = (r >> 6) & 3;
+    size_t kt = (r >> 8) % KT, item = (r >> 8) / KT;
+    const int tpm = 4 / s.nmat;
+    int mat = tile / tpm;
+    size_t row = item * s.rpi + (size_t)(tile % tpm) * 16 + (lane & 15);
+    const uint8_t* src = s.codes[mat] + (e * s.rows + row) * (s.K / 2) + kt * 64 + (lane >> 4) * 16;
+    dst[idx] = *reinterpret_cast<const uint4*>(src);
+}
+
+__global__ __launch_bounds__(256) void pack_scales_kernel(PackSrc s, int n_experts, uint32_t* __restrict__ dst) {
+    const int KT = s.K / 128, KT4 = (KT + 3) / 4;
+    const size_t items = s.rows / s.rpi;
+    const size_t per_expert = items * KT4 * 64 * 4;  // dwords per expert
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= per_expert * n_experts) return;
+    size_t e = idx / per_expert, r = idx % per_expert;
+    int tile = r & 3;
+    int lane = (r >> 2) & 63;
+    size_t k4 = (r >> 8) % KT4, item = (r >> 8) / KT4;
+    const int tpm = 4 / s.nmat;
+    int mat = tile / tpm;
+    size_t row = item * s.rpi + (size_t)(tile % tpm) * 16 + (lane & 15);
+    const uint8_t* src = s.scales[mat] + (e * s.rows + row) * (s.K / 32);
+    uint32_t v = 0;
+    for (int q = 0; q < 4; ++q) {
+        size_t kt = k4 * 4 + q;
+        uint32_t b = kt < (size_t)KT ? src[kt * 4 + (lane >> 4)] : 127u;
+        v |= b << (8 * q);
+    }
+    dst[idx] = v;
+}
+
+// ---- the streaming core ---------------------------------------------------------------------------
+// One wave, one item: for every k step, 4 A tiles from global memory (16 B per lane each), B from LDS, 4 MFMAs.
+// bq: [KT][2][64] uint4 (the unit's activations in operand order), bsc: [KT4][64] u32 (their scales).
+template <int Q>
+__device__ __forceinline__ void mfma_step(const u4v (&a)[4], const u4v& sc, const u4v* bq, uint32_t bscale,
+                                          int kt, int lane, v4f (&acc)[4]) {
+    const u4v b0 = bq[(kt * 2 + 0) * 64 + lane];
+    const u4v b1 = bq[(kt * 2 + 1) * 64 + lane];
+    const v8i bv = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+    const uint32_t scs[4] = {sc[0], sc[1], sc[2], sc[3]};
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const v8i av = {(int)a[t][0], (int)a[t][1], (int)a[t][2], (int)a[t][3], 0, 0, 0, 0};
+        acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[t], 4 /*A e2m1*/, 0 /*B e4m3*/, Q,
+                                                                  (int)scs[t], Q, (int)bscale);
+    }
+}
+
+__device__ __forceinline__ void stream_item(const u4v* __restrict__ wp, const u4v* __restrict__ sp, int KT,
+                                            const u4v* bq, const uint32_t* bsc, int lane, v4f (&acc)[4]) {
+    const int KT4 = (KT + 3) >> 2;
+    u4v a[2][4][4];   // [buffer][k step in group][tile]
+    u4v sc[2];
+    auto load_group = [&](int g4, int buf) {
+        sc[buf] = __builtin_nontemporal_load(&sp[(size_t)g4 * 64 + lane]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int kt = g4 * 4 + q;
+            if (kt < KT) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) a[buf][q][t] = __builtin_nontemporal_load(&wp[((size_t)kt * 4 + t) * 64 + lane]);
+            }
+        }
+    };
+    load_group(0, 0);
+    for (int g4 = 0; g4 < KT4; g4 += 2) {
+        if (g4 + 1 < KT4) load_group(g4 + 1, 1);
+        {
+            const uint32_t bs = bsc[g4 * 64 + lane];
+            const int kt = g4 * 4;
+            mfma_step<0>(a[0][0], sc[0], bq, bs, kt, lane, acc);
+            if (kt + 1 < KT) mfma_step<1>(a[0][1], sc[0], bq, bs, kt + 1, lane, acc);
+            if (kt + 2 < KT) mfma_step<2>(a[0][2], sc[0], bq, bs, kt + 2, lane, acc);
+            if (kt + 3 < KT) mfma_step<3>(a[0][3], sc[0], bq, bs, kt + 3, lane, acc);
+        }
+        if (g4 + 1 < KT4) {
+            if (g4 + 2 < KT4) load_group(g4 + 2, 0);
+            const uint32_t bs = bsc[(g4 + 1) * 64 + lane];
+            const int kt = (g4 + 1) * 4;
+            mfma_step<0>(a[1][0], sc[1], bq, bs, kt, lane, acc);
+            if (kt + 1 < KT) mfma_step<1>(a[1][1], sc[1], bq, bs, kt + 1, lane, acc);
+            if (kt + 2 < KT) mfma_step<2>(a[1][2], sc[1], bq, bs, kt + 2, lane, acc);
+            if (kt + 3 < KT) mfma_step<3>(a[1][3], sc[1], bq, bs, kt + 3, lane, acc);
+        }
+    }
+}
+
+// Copies the e4m3 rows of a unit into LDS in B-operand order and builds the packed scale words.
+// row_src(c) gives the source row index of column c (or -1).  q rows are K bytes, scale rows K/32 bytes.
+template <typename RowFn>
+__device__ __forceinline__ void fill_b_operand(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs, int K,
+                                               int nrows, RowFn row_src, u4v* bq, uint32_t* bsc) {
+    const int chunks = K / 16;
+    for (int idx = threadIdx.x; idx < nrows * chunks; idx += blockDim.x) {
+        const int c = idx / chunks, j = idx % chunks;
+        const int r = row_src(c);
+        u4v v = {0u, 0u, 0u, 0u};
+        if (r >= 0) v = *reinterpret_cast<const u4v*>(q + (size_t)r * K + (size_t)j * 16);
+        const int k = j * 16, kt = k >> 7, within = k & 127;
+        const int half = within >> 6, g = (within & 63) >> 4;
+        bq[(kt * 2 + half) * 64 + g * 16 + c] = v;
+    }
+    const int KT = K / 128, KT4 = (KT + 3) / 4;
+    for (int idx = threadIdx.x; idx < KT4 * 64; idx += blockDim.x) {
+        const int k4 = idx >> 6, l = idx & 63, c = l & 15, g = l >> 4;
+        uint32_t v = 0x7f7f7f7fu;
+        if (c < nrows) {
+            const int r = row_src(c);
+            if (r >= 0) {
+                v = 0;
+                for (int qq = 0; qq < 4; ++qq) {
+                    int kt = k4 * 4 + qq;
+                    uint32_t b = kt < KT ? qs[(size_t)r * (K / 32) + kt * 4 + g] : 127u;
+                    v |= b << (8 * qq);
+                }
+            }
+        }
+        bsc[idx] = v;
+    }
+}
+
+struct MfmaArgs {
+    const uint8_t* codes;         // routed experts
+    const uint8_t* scales;
+    const uint8_t* sh_codes;      // shared expert
+    const uint8_t* sh_scales;
+    size_t codes_per_expert, scales_per_expert;
+    const int32_t *unit_expert, *unit_row0, *unit_rows, *n_units;
+    int n, topk, n_experts, hidden, inter, shared_inter, act_ld;
+    float limit;
+};
+
+// gate/up GEMM + clamped SwiGLU + e4m3-per-32 quantisation of the result.
+// grid (ceil(items / WAVES), max_units); wave w of block b owns item b*WAVES + w of the unit's expert.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, const uint8_t* __restrict__ xq,
+                                                                  const uint8_t* __restrict__ xs,
+                                                                  const int32_t* __restrict__ gather_src,
+                                                                  uint8_t* __restrict__ act_q,
+                                                                  uint8_t* __restrict__ act_s) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    const int u = blockIdx.y;
+    if (u >= *a.n_units) return;
+    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    const bool shared = e == a.n_experts;
+    const int inter = shared ? a.shared_inter : a.inter;
+    const int items = inter / 32;
+    if ((int)blockIdx.x * WAVES >= items) return;
+    const int H = a.hidden, KT = H / 128, KT4 = (KT + 3) / 4;
+    u4v* bq = reinterpret_cast<u4v*>(lds_raw);
+    uint32_t* bsc = reinterpret_cast<uint32_t*>(lds_raw + (size_t)H * 16);
+    const int nk = a.n * a.topk, topk = a.topk;
+    auto row_src = [&](int c) -> int {
+        int g = row0 + c;
+        if (shared) return g - nk;
+        int i = gather_src[g];
+        return i < 0 ? -1 : i / topk;
+    };
+    fill_b_operand(xq, xs, H, nrows, row_src, bq, bsc);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int item = blockIdx.x * WAVES + wave;
+    if (item >= items) return;
+    const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
+    const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
+    const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
+    const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
+    v4f acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+    stream_item(wp, sp, KT, bq, bsc, lane, acc);
+
+    // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
+    float r0[4], r1[4];
+    float amax = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        r0[v] = swiglu_ref(acc[0][v], acc[2][v], a.limit);
+        r1[v] = swiglu_ref(acc[1][v], acc[3][v], a.limit);
+        amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+    }
+    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+    const int c = lane & 15, g = lane >> 4;
+    if (c < nrows) {
+        const uint32_t sb = block_scale_e8m0(amax);
+        const float inv = u2f((254u - sb) << 23);
+        uint32_t p0 = 0, p1 = 0;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            p0 |= e4m3_encode(r0[v] * inv) << (8 * v);
+            p1 |= e4m3_encode(r1[v] * inv) << (8 * v);
+        }
+        uint8_t* dst = act_q + (size_t)(row0 + c) * a.act_ld + (size_t)item * 32 + g * 4;
+        *reinterpret_cast<uint32_t*>(dst) = p0;
+        *reinterpret_cast<uint32_t*>(dst + 16) = p1;
+        if (g == 0) act_s[(size_t)(row0 + c) * (a.act_ld / 32) + item] = (uint8_t)sb;
+    }
+}
+
+// down GEMM: y[row][h] for the unit's rows.  grid (ceil(items / (WAVES*IPW)), max_units); item = 64 rows of H.
+template <int WAVES, int IPW>
+__global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const uint8_t* __restrict__ act_q,
+                                                               const uint8_t* __restrict__ act_s,
+                                                               float* __restrict__ y) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    const int u = blockIdx.y;
+    if (u >= *a.n_units) return;
+    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    const bool shared = e == a.n_experts;
+    const int inter = shared ? a.shared_inter : a.inter;
+    const int H = a.hidden, items = H / 64;
+    const int KT = inter / 128, KT4 = (KT + 3) / 4;
+    u4v* bq = reinterpret_cast<u4v*>(lds_raw);
+    uint32_t* bsc = reinterpret_cast<uint32_t*>(lds_raw + (size_t)a.act_ld * 16);
+    // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
+    {
+        const int chunks = inter / 16;
+        for (int idx = threadIdx.x; idx < nrows * chunks; idx += blockDim.x) {
+            const int c = idx / chunks, j = idx % chunks;
+            u4v v = *reinterpret_cast<const u4v*>(act_q + (size_t)(row0 + c) * a.act_ld + (size_t)j * 16);
+            const int k = j * 16, kt = k >> 7, within = k & 127;
+            bq[(kt * 2 + (within >> 6)) * 64 + ((within & 63) >> 4) * 16 + c] = v;
+        }
+        for (int idx = threadIdx.x; idx < KT4 * 64; idx += blockDim.x) {
+            const int k4 = idx >> 6, l = idx & 63, c = l & 15, g = l >> 4;
+            uint32_t v = 0x7f7f7f7fu;
+            if (c < nrows) {
+                v = 0;
+                for (int qq = 0; qq < 4; ++qq) {
+                    int kt = k4 * 4 + qq;
+                    uint32_t b = kt < KT ? act_s[(size_t)(row0 + c) * (a.act_ld / 32) + kt * 4 + g] : 127u;
+                    v |= b << (8 * qq);
+                }
+            }
+            bsc[idx] = v;
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
+    const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
+    const int c = lane & 15, g = lane >> 4;
+#pragma unroll 1
+    for (int ii = 0; ii < IPW; ++ii) {
+        const int item = (blockIdx.x * WAVES + wave) * IPW + ii;
+        if (item >= items) break;
+        const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
+        const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
+        v4f acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+        stream_item(wp, sp, KT, bq, bsc, lane, acc);
+        if (c < nrows) {
+            float* dst = y + (size_t)(row0 + c) * H + (size_t)item * 64 + g * 4;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                *reinterpret_cast<float4*>(dst + t * 16) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+        }
+    }
+}
+
+// ---- launchers ----------------------------------------------------------------------------------------
+constexpr int GU_WAVES = 4;
+constexpr int DN_WAVES = 4;
+constexpr int DN_IPW = 2;
+
+static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int n, const UnitTables& units, bool down) {
+    PackedLayout L = packed_layout(s);
+    MfmaArgs a{};
+    a.codes = packed + (down ? L.dn_codes : L.gu_codes);
+    a.scales = packed + (down ? L.dn_scales : L.gu_scales);
+    a.sh_codes = packed + (down ? L.sh_dn_codes : L.sh_gu_codes);
+    a.sh_scales = packed + (down ? L.sh_dn_scales : L.sh_gu_scales);
+    a.codes_per_expert = down ? L.dn_codes_per_expert : L.gu_codes_per_expert;
+    a.scales_per_expert = down ? L.dn_scales_per_expert : L.gu_scales_per_expert;
+    a.unit_expert = units.unit_expert; a.unit_row0 = units.unit_row0; a.unit_rows = units.unit_rows;
+    a.n_units = units.n_units;
+    a.n = n; a.topk = s.topk; a.n_experts = s.n_experts; a.hidden = s.hidden; a.inter = s.inter;
+    a.shared_inter = s.shared_inter;
+    a.act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
+    a.limit = s.swiglu_limit;
+    return a;
+}
+
+// Kernels that need more than 64 KiB of dynamic LDS must have the limit raised once (a function attribute,
+// not a stream operation).  `raised` remembers the largest value already set for that kernel.
+template <typename K>
+static int set_lds_limit(K kernel, size_t bytes, size_t* raised) {
+    if (bytes <= 64 * 1024 || bytes <= *raised) return FERRITE_OK;
+    if (bytes > 160 * 1024) return FERRITE_DECLINED;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+    *raised = bytes;
+    return FERRITE_OK;
+}
+
+int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
+                        int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
+                        hipStream_t st) {
+    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
+    MfmaArgs a = make_args(s, packed, n, units, false);
+    const int imax = a.act_ld;
+    const size_t lds = (size_t)s.hidden * 16 + (size_t)((s.hidden / 128 + 3) / 4) * 256;
+    static size_t raised = 0;
+    int rc = set_lds_limit(gate_up_mfma_kernel<GU_WAVES>, lds, &raised);
+    if (rc) return rc;
+    dim3 grid((imax / 32 + GU_WAVES - 1) / GU_WAVES, units.max_units);
+    gate_up_mfma_kernel<GU_WAVES><<<grid, GU_WAVES * 64, lds, st>>>(a, xq, xs, gather_src, act_q, act_s);
+    return check_launch("gate_up_mfma");
+}
+
+int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
+                     int n, const UnitTables& units, float* y, hipStream_t st) {
+    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
+    MfmaArgs a = make_args(s, packed, n, units, true);
+    const size_t lds = (size_t)a.act_ld * 16 + (size_t)((a.act_ld / 128 + 3) / 4) * 256;
+    static size_t raised = 0;
+    int rc = set_lds_limit(down_mfma_kernel<DN_WAVES, DN_IPW>, lds, &raised);
+    if (rc) return rc;
+    const int items = s.hidden / 64;
+    dim3 grid((items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW), units.max_units);
+    down_mfma_kernel<DN_WAVES, DN_IPW><<<grid, DN_WAVES * 64, lds, st>>>(a, act_q, act_s, y);
+    return check_launch("down_mfma");
+}
+
+}  // namespace fe
+
+using namespace fe;
+
+static int check_shape_mfma(const ferrite_moe_shape* s) {
+    if (!s) return FERRITE_ERR_INVALID_ARG;
+    if (s->hidden <= 0 || s->inter <= 0 || s->n_experts <= 0 || s->shared_inter < 0) return FERRITE_ERR_INVALID_ARG;
+    if (s->hidden % 128 || s->inter % 128 || s->shared_inter % 128) return FERRITE_DECLINED;
+    return FERRITE_OK;
+}
+
+extern "C" size_t ferrite_moe_packed_bytes(const ferrite_moe_shape* shape) {
+    if (check_shape_mfma(shape)) return 0;
+    return packed_layout(*shape).total;
+}
+
+static int pack_one(const PackSrc& src, int n_experts, uint8_t* codes_dst, uint8_t* scales_dst, hipStream_t st) {
+    if (src.rows == 0 || n_experts == 0) return FERRITE_OK;
+    const size_t KT = src.K / 128, KT4 = (KT + 3) / 4, items = src.rows / src.rpi;
+    size_t nc = items * KT * 256 * n_experts;
+    pack_codes_kernel<<<(unsigned)((nc + 255) / 256), 256, 0, st>>>(src, n_experts, reinterpret_cast<uint4*>(codes_dst));
+    int rc = check_launch("pack_codes");
+    if (rc) return rc;
+    size_t ns = items * KT4 * 256 * n_experts;
+    pack_scales_kernel<<<(unsigned)((ns + 255) / 256), 256, 0, st>>>(src, n_experts, reinterpret_cast<uint32_t*>(scales_dst));
+    return check_launch("pack_scales");
+}
+
+extern "C" int ferrite_moe_pack_weights(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, uint8_t* packed,
+                                        ferrite_stream_t stream) {
+    int rc = check_shape_mfma(shape);
+    if (rc) return rc;
+    if (!w || !packed || !w->gate_w || !w->gate_s || !w->up_w || !w->up_s || !w->down_w || !w->down_s)
+        return FERRITE_ERR_INVALID_ARG;
+    if (shape->shared_inter > 0 && (!w->sh_gate_w || !w->sh_gate_s || !w->sh_up_w || !w->sh_up_s || !w->sh_down_w || !w->sh_down_s))
+        return FERRITE_ERR_INVALID_ARG;
+    const ferrite_moe_shape& s = *shape;
+    PackedLayout L = packed_layout(s);
+    hipStream_t st = as_stream(stream);
+    PackSrc gu{{w->gate_w, w->up_w}, {w->gate_s, w->up_s}, s.inter, s.hidden, 2, 32};
+    if ((rc = pack_one(gu, s.n_experts, packed + L.gu_codes, packed + L.gu_scales, st))) return rc;
+    PackSrc dn{{w->down_w, nullptr}, {w->down_s, nullptr}, s.hidden, s.inter, 1, 64};
+    if ((rc = pack_one(dn, s.n_experts, packed + L.dn_codes, packed + L.dn_scales, st))) return rc;
+    if (s.shared_inter > 0) {
+        PackSrc sgu{{w->sh_gate_w, w->sh_up_w}, {w->sh_gate_s, w->sh_up_s}, s.shared_inter, s.hidden, 2, 32};
+        if ((rc = pack_one(sgu, 1, packed + L.sh_gu_codes, packed + L.sh_gu_scales, st))) return rc;
+        PackSrc sdn{{w->sh_down_w, nullptr}, {w->sh_down_s, nullptr}, s.hidden, s.shared_inter, 1, 64};
+        if ((rc = pack_one(sdn, 1, packed + L.sh_dn_codes, packed + L.sh_dn_scales, st))) return rc;
+    }
+    return FERRITE_OK;
+}
+
+// dequantise one matrix out of the packed buffer (verification of the permutation)
+__global__ __launch_bounds__(256) void packed_dequant_kernel(const uint4* __restrict__ codes,
+                                                             const uint32_t* __restrict__ scales, int rows, int K,
+                                                             int nmat, int rpi, int mat, float* __restrict__ dst) {
+    // one thread per (row, 32-column block)
+    const int KT = K / 128, KT4 = (KT + 3) / 4;
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)rows * (K / 32)) return;
+    int row = (int)(idx / (K / 32)), kb = (int)(idx % (K / 32));
+    int kt = kb >> 2, g = kb & 3;
+    int item = row / rpi, rin = row % rpi;
+    const int tpm = 4 / nmat;
+    int tile = mat * tpm + rin / 16, lane = g * 16 + (rin & 15);
+    uint4 c = codes[(((size_t)item * KT + kt) * 4 + tile) * 64 + lane];
+    uint32_t sw = scales[(((size_t)item * KT4 + (kt >> 2)) * 64 + lane) * 4 + tile];
+    float s = fe::ue8m0_decode((sw >> (8 * (kt & 3))) & 0xffu);
+    uint32_t words[4] = {c.x, c.y, c.z, c.w};
+    float* o = dst + (size_t)row * K + (size_t)kb * 32;
+    for (int q = 0; q < 4; ++q)
+        for (int b = 0; b < 8; ++b) o[q * 8 + b] = fe::e2m1_decode((words[q] >> (4 * b)) & 15u) * s;
+}
+
+extern "C" int ferrite_moe_packed_dequant(const ferrite_moe_shape* shape, const uint8_t* packed, int expert, int which,
+                                          float* dst, ferrite_stream_t stream) {
+    int rc = check_shape_mfma(shape);
+    if (rc) return rc;
+    const ferrite_moe_shape& s = *shape;
+    if (!packed || !dst || which < 0 || which > 2 || expert < 0 || expert > s.n_experts) return FERRITE_ERR_INVALID_ARG;
+    const bool shared = expert == s.n_experts;
+    if (shared && s.shared_inter == 0) return FERRITE_ERR_INVALID_ARG;
+    PackedLayout L = packed_layout(s);
+    const int inter = shared ? s.shared_inter : s.inter;
+    const bool down = which == 2;
+    const int rows = down ? s.hidden : inter, K = down ? inter : s.hidden;
+    const size_t KT = K / 128, KT4 = (KT + 3) / 4;
+    const int rpi = down ? 64 : 32, nmat = down ? 1 : 2;
+    const size_t items = rows / rpi;
+    const size_t cpe = items * KT * 4096, spe = items * KT4 * 1024;
+    const uint8_t* cb = packed + (shared ? (down ? L.sh_dn_codes : L.sh_gu_codes)
+                                         : (down ? L.dn_codes : L.gu_codes) + (size_t)expert * cpe);
+    const uint8_t* sb = packed + (shared ? (down ? L.sh_dn_scales : L.sh_gu_scales)
+                                         : (down ? L.dn_scales : L.gu_scales) + (size_t)expert * spe);
+    size_t total = (size_t)rows * (K / 32);
+    packed_dequant_kernel<<<(unsigned)((total + 255) / 256), 256, 0, as_stream(stream)>>>(
+        reinterpret_cast<const uint4*>(cb), reinterpret_cast<const uint32_t*>(sb), rows, K, nmat, rpi, down ? 0 : which, dst);
+    return check_launch("packed_dequant");
+}

@@ -1,0 +1,111 @@
+// MXFP4 -> f32 dequantisation and e4m3-per-32 activation quantisation.  Both are bit-exact restatements of
+// crates/ferrite-models/src/dsv41/quant.rs (dequant_fp4_row32 :260-278, act_quant_fp8 :190-214) and are
+// bound by HBM traffic: every thread moves 128-bit vectors.
+#include "internal.hpp"
+#include "numerics.hpp"
+
+namespace fe {
+
+// One thread dequantises 32 columns of one row: 16 code bytes (one 128-bit load) and one scale byte in,
+// 32 floats (eight 128-bit stores) out.
+__global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t* __restrict__ w,
+                                                            const uint8_t* __restrict__ scale, int64_t nblocks,
+                                                            float* __restrict__ dst) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    uint4 c = *reinterpret_cast<const uint4*>(w + b * 16);
+    float s = ue8m0_decode(scale[b]);
+    uint32_t words[4] = {c.x, c.y, c.z, c.w};
+    float4* o = reinterpret_cast<float4*>(dst + b * 32);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t v = words[q];
+        float4 lo, hi;
+        lo.x = e2m1_decode(v & 15u) * s;         lo.y = e2m1_decode((v >> 4) & 15u) * s;
+        lo.z = e2m1_decode((v >> 8) & 15u) * s;  lo.w = e2m1_decode((v >> 12) & 15u) * s;
+        hi.x = e2m1_decode((v >> 16) & 15u) * s; hi.y = e2m1_decode((v >> 20) & 15u) * s;
+        hi.z = e2m1_decode((v >> 24) & 15u) * s; hi.w = e2m1_decode((v >> 28) & 15u) * s;
+        o[2 * q] = lo;
+        o[2 * q + 1] = hi;
+    }
+}
+
+// One thread quantises one block of 32 consecutive values of a row.
+template <typename XT>
+__global__ __launch_bounds__(256) void act_quant_kernel(const XT* __restrict__ x, int64_t nblocks,
+                                                        uint8_t* __restrict__ q, uint8_t* __restrict__ scale) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    float v[32];
+    if constexpr (sizeof(XT) == 4) {
+        const float4* p = reinterpret_cast<const float4*>(x + b * 32);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float4 t = p[i];
+            v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+        }
+    } else {
+        const uint4* p = reinterpret_cast<const uint4*>(x + b * 32);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4 t = p[i];
+            uint32_t wds[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[8 * i + 2 * j] = u2f(wds[j] << 16);
+                v[8 * i + 2 * j + 1] = u2f(wds[j] & 0xffff0000u);
+            }
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    uint32_t sb = block_scale_e8m0(amax);
+    float inv = u2f((254u - sb) << 23);   // 2^(127 - sb): exact reciprocal of the power-of-two scale
+    uint32_t out[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        out[i] = e4m3_encode(v[4 * i] * inv) | (e4m3_encode(v[4 * i + 1] * inv) << 8) |
+                 (e4m3_encode(v[4 * i + 2] * inv) << 16) | (e4m3_encode(v[4 * i + 3] * inv) << 24);
+    }
+    uint4* o = reinterpret_cast<uint4*>(q + b * 32);
+    o[0] = make_uint4(out[0], out[1], out[2], out[3]);
+    o[1] = make_uint4(out[4], out[5], out[6], out[7]);
+    scale[b] = (uint8_t)sb;
+}
+
+int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, hipStream_t st) {
+    if (rows < 0 || cols < 0 || cols % 32 != 0) return FERRITE_ERR_INVALID_ARG;
+    int64_t nblocks = rows * (cols / 32);
+    if (nblocks == 0) return FERRITE_OK;
+    unsigned grid = (unsigned)((nblocks + 255) / 256);
+    if (x_dtype == FERRITE_DT_F32)
+        act_quant_kernel<float><<<grid, 256, 0, st>>>((const float*)x, nblocks, q, scale);
+    else if (x_dtype == FERRITE_DT_BF16)
+        act_quant_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)x, nblocks, q, scale);
+    else
+        return FERRITE_ERR_INVALID_ARG;
+    return check_launch("act_quant");
+}
+
+}  // namespace fe
+
+using namespace fe;
+
+extern "C" int ferrite_mxfp4_dequant(const uint8_t* w, const uint8_t* scale, int64_t rows, int64_t cols, float* dst,
+                                     ferrite_stream_t stream) {
+    if (rows < 0 || cols < 0 || cols % 32 != 0) return FERRITE_ERR_INVALID_ARG;
+    int64_t nblocks = rows * (cols / 32);
+    if (nblocks == 0) return FERRITE_OK;
+    if (!w || !scale || !dst) return FERRITE_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(w) & 15) || (reinterpret_cast<uintptr_t>(dst) & 15)) return FERRITE_DECLINED;
+    mxfp4_dequant_kernel<<<(unsigned)((nblocks + 255) / 256), 256, 0, as_stream(stream)>>>(w, scale, nblocks, dst);
+    return check_launch("mxfp4_dequant");
+}
+
+extern "C" int ferrite_act_quant_fp8(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale,
+                                     ferrite_stream_t stream) {
+    if (rows > 0 && cols > 0 && (!x || !q || !scale)) return FERRITE_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(q) & 15)) return FERRITE_DECLINED;
+    return launch_act_quant(x, x_dtype, rows, cols, q, scale, as_stream(stream));
+}

@@ -1,0 +1,69 @@
+// Declarations shared between the translation units of libferrite_hip.so (not part of the public ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/ferrite_hip.h"
+
+namespace fe {
+
+// Records a failed HIP runtime call for ferrite_hip_last_error() and returns FERRITE_ERR_RUNTIME.
+int hip_fail(hipError_t e, const char* what);
+// Checks the launch that was just issued on this thread.
+int check_launch(const char* what);
+
+inline hipStream_t as_stream(ferrite_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// A unit is up to `unit_rows` consecutive rows of the grouped order that share one expert; the expert GEMM
+// kernels are launched over a fixed upper bound of units and read the live count from n_units.
+struct UnitTables {
+    int32_t* unit_expert;  // [max_units] expert id (n_experts = the shared expert)
+    int32_t* unit_row0;    // [max_units] first grouped row
+    int32_t* unit_rows;    // [max_units] rows in the unit (1..unit_rows)
+    int32_t* n_units;      // [1]
+    int unit_rows_cap;     // rows per unit (column tile of the GEMM)
+    int max_units;
+};
+
+inline int max_units_for(int n, int topk, int n_experts, int has_shared, int unit_rows) {
+    long assign = (long)n * topk;
+    long active_max = assign < n_experts ? assign : n_experts;
+    long u = assign / unit_rows + active_max + (has_shared ? (n + unit_rows - 1) / unit_rows : 0);
+    return (int)u;
+}
+
+// route.hip
+int launch_matmul_exact(const void* x, int x_dtype, const float* w, const float* bias, float* out, int n, int k,
+                        int o, hipStream_t st);
+int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* counts, int32_t* starts,
+                   int32_t* perm_map, int32_t* gather_src, int32_t* active, int32_t* n_active, void* scratch,
+                   size_t scratch_bytes, const UnitTables* units, int has_shared, hipStream_t st);
+
+// experts_f32.hip (check mode)
+int launch_gate_up_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, const float* x, int n,
+                       const int32_t* ids, const int32_t* gather_src, float* act, hipStream_t st);
+int launch_down_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, const float* act, int n,
+                    const int32_t* ids, const int32_t* gather_src, float* y, hipStream_t st);
+int launch_combine(const float* y, const float* probs, const int32_t* perm_map, int n, int topk, int hidden,
+                   int has_shared, void* out, int out_dtype, hipStream_t st);
+
+// experts_mfma.hip
+struct PackedLayout {
+    // byte offsets into the packed buffer
+    size_t gu_codes, gu_scales, dn_codes, dn_scales;           // routed experts
+    size_t sh_gu_codes, sh_gu_scales, sh_dn_codes, sh_dn_scales; // shared expert
+    size_t gu_codes_per_expert, gu_scales_per_expert, dn_codes_per_expert, dn_scales_per_expert;
+    size_t total;
+};
+PackedLayout packed_layout(const ferrite_moe_shape& s);
+int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
+                        int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
+                        hipStream_t st);
+int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
+                     int n, const UnitTables& units, float* y, hipStream_t st);
+
+// formats.hip
+int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, hipStream_t st);
+
+}  // namespace fe

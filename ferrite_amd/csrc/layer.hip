@@ -1,0 +1,226 @@
+// Library identity, error reporting, workspace carving, the fused MoE layer driver and the graph entry points.
+// The driver only enqueues kernels on the caller's stream: no allocation, no synchronisation, no host reads
+// of device data, and a launch sequence that is a function of (shape, n, mode) alone.
+#include <stdio.h>
+#include <string.h>
+
+#include "internal.hpp"
+
+#ifndef FERRITE_BUILD_ID
+#define FERRITE_BUILD_ID "unstamped"
+#endif
+
+namespace fe {
+
+static thread_local char g_last_error[256] = "";
+
+int hip_fail(hipError_t e, const char* what) {
+    snprintf(g_last_error, sizeof(g_last_error), "HIP %s: %s", what, hipGetErrorString(e));
+    return FERRITE_ERR_RUNTIME;
+}
+
+int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(e, what);
+    return FERRITE_OK;
+}
+
+// ---- workspace: fixed offsets for (shape, n, mode) ----
+struct Workspace {
+    size_t logits, probs, ids_f32, ids, counts, starts, perm_map, gather_src, active, n_active;
+    size_t unit_expert, unit_row0, unit_rows, n_units, perm_scratch, perm_scratch_bytes;
+    size_t xq, xs, act, act_s, y;
+    size_t total;
+    int max_units, rows;
+};
+
+static size_t bump(size_t& off, size_t bytes) {
+    size_t at = off;
+    off = (off + bytes + 255) / 256 * 256;
+    return at;
+}
+
+static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
+    Workspace w{};
+    const size_t nk = (size_t)n * s.topk, E = s.n_experts, H = s.hidden;
+    const int has_shared = s.shared_inter > 0;
+    const size_t act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
+    w.rows = (int)(nk + (has_shared ? n : 0));
+    w.max_units = max_units_for(n, s.topk, s.n_experts, has_shared, 16);
+    size_t off = 0;
+    w.logits = bump(off, (size_t)n * E * 4);
+    w.probs = bump(off, nk * 4);
+    w.ids_f32 = bump(off, nk * 4);
+    w.ids = bump(off, nk * 4);
+    w.counts = bump(off, E * 4);
+    w.starts = bump(off, (E + 1) * 4);
+    w.perm_map = bump(off, nk * 4);
+    w.gather_src = bump(off, nk * 4);
+    w.active = bump(off, E * 4);
+    w.n_active = bump(off, 4);
+    w.unit_expert = bump(off, (size_t)w.max_units * 4);
+    w.unit_row0 = bump(off, (size_t)w.max_units * 4);
+    w.unit_rows = bump(off, (size_t)w.max_units * 4);
+    w.n_units = bump(off, 4);
+    w.perm_scratch_bytes = ferrite_moe_permute_scratch_bytes(n, s.n_experts);
+    w.perm_scratch = bump(off, w.perm_scratch_bytes);
+    if (mode == FERRITE_MODE_MFMA_FP8) {
+        w.xq = bump(off, (size_t)n * H);
+        w.xs = bump(off, (size_t)n * (H / 32));
+        w.act = bump(off, (size_t)w.rows * act_ld);
+        w.act_s = bump(off, (size_t)w.rows * (act_ld / 32));
+    } else {
+        w.act = bump(off, (size_t)w.rows * act_ld * 4);
+    }
+    w.y = bump(off, (size_t)w.rows * H * 4);
+    w.total = off;
+    return w;
+}
+
+static int check_shape(const ferrite_moe_shape* s, int n, int mode) {
+    if (!s || n <= 0) return FERRITE_ERR_INVALID_ARG;
+    if (s->hidden <= 0 || s->n_experts <= 0 || s->topk <= 0 || s->topk > s->n_experts || s->inter <= 0 ||
+        s->shared_inter < 0)
+        return FERRITE_ERR_INVALID_ARG;
+    if (mode != FERRITE_MODE_F32_CHECK && mode != FERRITE_MODE_MFMA_FP8) return FERRITE_ERR_INVALID_ARG;
+    if (s->hidden % 32 || s->inter % 32 || s->shared_inter % 32) return FERRITE_ERR_INVALID_ARG;
+    if (mode == FERRITE_MODE_MFMA_FP8 && (s->hidden % 128 || s->inter % 128 || s->shared_inter % 128))
+        return FERRITE_DECLINED;
+    if ((long long)n * s->topk > 0x7fffffffLL / 2) return FERRITE_DECLINED;
+    return FERRITE_OK;
+}
+
+}  // namespace fe
+
+using namespace fe;
+
+extern "C" const char* ferrite_kernel_build_id(void) { return FERRITE_BUILD_ID; }
+extern "C" unsigned ferrite_kernel_abi_version(void) { return FERRITE_ABI_VERSION; }
+extern "C" const char* ferrite_hip_last_error(void) { return g_last_error; }
+
+extern "C" size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode) {
+    if (check_shape(shape, n, mode)) return 0;
+    return carve(*shape, n, mode).total;
+}
+
+extern "C" int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int mode, void* workspace,
+                                                ferrite_moe_workspace_view* v) {
+    int rc = check_shape(shape, n, mode);
+    if (rc) return rc;
+    if (!workspace || !v) return FERRITE_ERR_INVALID_ARG;
+    Workspace w = carve(*shape, n, mode);
+    char* b = static_cast<char*>(workspace);
+    v->logits = reinterpret_cast<float*>(b + w.logits);
+    v->probs = reinterpret_cast<float*>(b + w.probs);
+    v->ids_f32 = reinterpret_cast<float*>(b + w.ids_f32);
+    v->ids = reinterpret_cast<int32_t*>(b + w.ids);
+    v->counts = reinterpret_cast<int32_t*>(b + w.counts);
+    v->starts = reinterpret_cast<int32_t*>(b + w.starts);
+    v->perm_map = reinterpret_cast<int32_t*>(b + w.perm_map);
+    v->gather_src = reinterpret_cast<int32_t*>(b + w.gather_src);
+    v->active = reinterpret_cast<int32_t*>(b + w.active);
+    v->n_active = reinterpret_cast<int32_t*>(b + w.n_active);
+    v->y = reinterpret_cast<float*>(b + w.y);
+    return FERRITE_OK;
+}
+
+extern "C" int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
+                                       const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
+                                       int out_dtype, int mode, void* workspace, size_t workspace_bytes,
+                                       ferrite_stream_t stream) {
+    int rc = check_shape(shape, n, mode);
+    if (rc) return rc;
+    if (!wts || !wts->router_w || !x || !out || !workspace) return FERRITE_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255) || (reinterpret_cast<uintptr_t>(x) & 15) ||
+        (reinterpret_cast<uintptr_t>(out) & 15))
+        return FERRITE_ERR_INVALID_ARG;
+    if (x_dtype != FERRITE_DT_F32 && x_dtype != FERRITE_DT_BF16) return FERRITE_ERR_INVALID_ARG;
+    if (out_dtype != FERRITE_DT_F32 && out_dtype != FERRITE_DT_BF16) return FERRITE_ERR_INVALID_ARG;
+    const ferrite_moe_shape& s = *shape;
+    if (mode == FERRITE_MODE_F32_CHECK) {
+        if (x_dtype != FERRITE_DT_F32) return FERRITE_ERR_INVALID_ARG;
+        if (!wts->gate_w || !wts->gate_s || !wts->up_w || !wts->up_s || !wts->down_w || !wts->down_s)
+            return FERRITE_ERR_INVALID_ARG;
+        if (s.shared_inter > 0 && (!wts->sh_gate_w || !wts->sh_gate_s || !wts->sh_up_w || !wts->sh_up_s ||
+                                   !wts->sh_down_w || !wts->sh_down_s))
+            return FERRITE_ERR_INVALID_ARG;
+    } else if (!packed) {
+        return FERRITE_ERR_INVALID_ARG;
+    }
+    Workspace w = carve(s, n, mode);
+    if (workspace_bytes < w.total) return FERRITE_ERR_WORKSPACE;
+    char* b = static_cast<char*>(workspace);
+    hipStream_t st = as_stream(stream);
+    const int has_shared = s.shared_inter > 0;
+
+    float* logits = reinterpret_cast<float*>(b + w.logits);
+    float* probs = reinterpret_cast<float*>(b + w.probs);
+    float* ids_f32 = reinterpret_cast<float*>(b + w.ids_f32);
+    int32_t* ids = reinterpret_cast<int32_t*>(b + w.ids);
+    int32_t* perm_map = reinterpret_cast<int32_t*>(b + w.perm_map);
+    int32_t* gather_src = reinterpret_cast<int32_t*>(b + w.gather_src);
+    float* y = reinterpret_cast<float*>(b + w.y);
+
+    // 1. router logits: the reference's sequential-k f32 chain (exec/lib.rs:1107)
+    if ((rc = launch_matmul_exact(x, x_dtype, wts->router_w, nullptr, logits, n, s.hidden, s.n_experts, st))) return rc;
+    // 2. routing (exec/lib.rs:1109-1116); a NULL bias is the reference's zero bias
+    if ((rc = ferrite_moe_route(logits, wts->router_bias, n, s.n_experts, s.topk, s.n_group, s.topk_group,
+                                s.routed_scaling, probs, ids_f32, ids, stream)))
+        return rc;
+    // 3. permutation by expert + unit tables
+    UnitTables units{reinterpret_cast<int32_t*>(b + w.unit_expert), reinterpret_cast<int32_t*>(b + w.unit_row0),
+                     reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.n_units), 16,
+                     w.max_units};
+    if ((rc = launch_permute(ids, n, s.topk, s.n_experts, reinterpret_cast<int32_t*>(b + w.counts),
+                             reinterpret_cast<int32_t*>(b + w.starts), perm_map, gather_src,
+                             reinterpret_cast<int32_t*>(b + w.active), reinterpret_cast<int32_t*>(b + w.n_active),
+                             b + w.perm_scratch, w.perm_scratch_bytes, &units, has_shared, st)))
+        return rc;
+    // 4-5. expert FFNs in grouped order, shared expert as the trailing rows
+    if (mode == FERRITE_MODE_F32_CHECK) {
+        float* act = reinterpret_cast<float*>(b + w.act);
+        if ((rc = launch_gate_up_f32(s, *wts, static_cast<const float*>(x), n, ids, gather_src, act, st))) return rc;
+        if ((rc = launch_down_f32(s, *wts, act, n, ids, gather_src, y, st))) return rc;
+    } else {
+        uint8_t* xq = reinterpret_cast<uint8_t*>(b + w.xq);
+        uint8_t* xs = reinterpret_cast<uint8_t*>(b + w.xs);
+        uint8_t* act_q = reinterpret_cast<uint8_t*>(b + w.act);
+        uint8_t* act_s = reinterpret_cast<uint8_t*>(b + w.act_s);
+        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq, xs, st))) return rc;
+        if ((rc = launch_gate_up_mfma(s, packed, xq, xs, n, gather_src, units, act_q, act_s, st))) return rc;
+        if ((rc = launch_down_mfma(s, packed, act_q, act_s, n, units, y, st))) return rc;
+    }
+    // 6. weighted combine in slot order + shared expert (exec/lib.rs:1154-1164)
+    return launch_combine(y, probs, perm_map, n, s.topk, s.hidden, has_shared, out, out_dtype, st);
+}
+
+// ---- graph capture (ferrite_graph_begin/end/instantiate/launch, cuda.rs:284-287) ----
+extern "C" int ferrite_graph_begin(ferrite_stream_t stream) {
+    hipError_t e = hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal);
+    return e == hipSuccess ? FERRITE_OK : hip_fail(e, "hipStreamBeginCapture");
+}
+
+extern "C" int ferrite_graph_end(ferrite_stream_t stream, void** graph_exec_out) {
+    if (!graph_exec_out) return FERRITE_ERR_INVALID_ARG;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(as_stream(stream), &graph);
+    if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture");
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    hipGraphDestroy(graph);
+    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    *graph_exec_out = exec;
+    return FERRITE_OK;
+}
+
+extern "C" int ferrite_graph_launch(void* graph_exec, ferrite_stream_t stream) {
+    if (!graph_exec) return FERRITE_ERR_INVALID_ARG;
+    hipError_t e = hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), as_stream(stream));
+    return e == hipSuccess ? FERRITE_OK : hip_fail(e, "hipGraphLaunch");
+}
+
+extern "C" int ferrite_graph_destroy(void* graph_exec) {
+    if (!graph_exec) return FERRITE_OK;
+    hipError_t e = hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec));
+    return e == hipSuccess ? FERRITE_OK : hip_fail(e, "hipGraphExecDestroy");
+}

@@ -1,0 +1,561 @@
+// Router logits (bit-exact sequential-k f32 GEMM), noaux-tc sigmoid group-limited top-k, and the stable
+// token permutation by expert.  gfx950, wave64.
+#include "internal.hpp"
+#include "numerics.hpp"
+
+namespace fe {
+
+// ------------------------------------------------------------------------------------------------
+// x . w^T with the reference's arithmetic (crates/ferrite-kernel/src/cpu.rs:106-111): for every output one
+// chain s = 0; s = fl(s + fl(x[l] * w[l])) in ascending l.  The chain cannot be re-associated, so the
+// kernel gives every output its own lane and only organises the operand traffic: a block owns 4 rows of x
+// and 64 rows of w, stages 64-wide k-chunks of both through LDS (w transposed so that a lane reads four
+// consecutive k of its own row with one 128-bit LDS read), and double-buffers the staging.
+// ------------------------------------------------------------------------------------------------
+constexpr int MM_TT = 4;    // x rows per block (one per wave)
+constexpr int MM_TO = 64;   // w rows per block (one per lane)
+constexpr int MM_KC = 64;   // k chunk
+constexpr int MM_WPAD = MM_TO + 1;
+
+__device__ __forceinline__ float load_x(const float* p, size_t i) { return p[i]; }
+__device__ __forceinline__ float load_x(const uint16_t* p, size_t i) { return u2f((uint32_t)p[i] << 16); }
+
+template <typename XT>
+__global__ __launch_bounds__(256) void matmul_exact_kernel(const XT* __restrict__ x, const float* __restrict__ w,
+                                                           const float* __restrict__ bias, float* __restrict__ out,
+                                                           int n, int k, int o) {
+    __shared__ float4 w_lds[2][MM_KC / 4][MM_WPAD];
+    __shared__ float4 x_lds[2][MM_TT][MM_KC / 4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int o0 = blockIdx.x * MM_TO, t0 = blockIdx.y * MM_TT;
+    const int nchunk = (k + MM_KC - 1) / MM_KC;
+
+    // staging assignment: 64 w rows x 16 float4 per chunk = 1024 float4 -> 4 per thread; x: 4 x 16 = 64 float4
+    float4 wreg[4];
+    float4 xreg;
+    auto fetch = [&](int c) {
+        const int kb = c * MM_KC;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            int idx = tid + p * 256;
+            int r = idx >> 4, c4 = idx & 15;
+            int col = kb + c4 * 4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (o0 + r < o) {
+                const float* src = w + (size_t)(o0 + r) * k + col;
+                if (col + 3 < k) v = *reinterpret_cast<const float4*>(src);
+                else {
+                    if (col < k) v.x = src[0];
+                    if (col + 1 < k) v.y = src[1];
+                    if (col + 2 < k) v.z = src[2];
+                }
+            }
+            wreg[p] = v;
+        }
+        if (tid < MM_TT * (MM_KC / 4)) {
+            int r = tid >> 4, c4 = tid & 15;
+            int col = kb + c4 * 4;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (t0 + r < n) {
+                size_t base = (size_t)(t0 + r) * k + col;
+                if (col < k) v.x = load_x(x, base);
+                if (col + 1 < k) v.y = load_x(x, base + 1);
+                if (col + 2 < k) v.z = load_x(x, base + 2);
+                if (col + 3 < k) v.w = load_x(x, base + 3);
+            }
+            xreg = v;
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            int idx = tid + p * 256;
+            int r = idx >> 4, c4 = idx & 15;
+            w_lds[buf][c4][r] = wreg[p];
+        }
+        if (tid < MM_TT * (MM_KC / 4)) x_lds[buf][tid >> 4][tid & 15] = xreg;
+    };
+
+    float s = 0.0f;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int c = 0; c < nchunk; ++c) {
+        const int buf = c & 1;
+        if (c + 1 < nchunk) fetch(c + 1);
+        const int klen = min(MM_KC, k - c * MM_KC);
+        const int full4 = klen >> 2;
+        for (int c4 = 0; c4 < full4; ++c4) {
+            float4 wv = w_lds[buf][c4][lane];
+            float4 xv = x_lds[buf][wave][c4];
+            s = fadd(s, fmul(xv.x, wv.x));
+            s = fadd(s, fmul(xv.y, wv.y));
+            s = fadd(s, fmul(xv.z, wv.z));
+            s = fadd(s, fmul(xv.w, wv.w));
+        }
+        if (klen & 3) {
+            float4 wv = w_lds[buf][full4][lane];
+            float4 xv = x_lds[buf][wave][full4];
+            int rem = klen & 3;
+            s = fadd(s, fmul(xv.x, wv.x));
+            if (rem > 1) s = fadd(s, fmul(xv.y, wv.y));
+            if (rem > 2) s = fadd(s, fmul(xv.z, wv.z));
+        }
+        if (c + 1 < nchunk) stash(buf ^ 1);
+        __syncthreads();
+    }
+    const int t = t0 + wave, j = o0 + lane;
+    if (t < n && j < o) {
+        if (bias) s = fadd(s, bias[j]);
+        out[(size_t)t * o + j] = s;
+    }
+}
+
+int launch_matmul_exact(const void* x, int x_dtype, const float* w, const float* bias, float* out, int n, int k,
+                        int o, hipStream_t st) {
+    if (n < 0 || k < 0 || o < 0) return FERRITE_ERR_INVALID_ARG;
+    if (n == 0 || o == 0) return FERRITE_OK;
+    dim3 grid((o + MM_TO - 1) / MM_TO, (n + MM_TT - 1) / MM_TT);
+    // the staging reads w with 128-bit loads: row starts must be 16-byte aligned
+    if ((k & 3) != 0 || (reinterpret_cast<uintptr_t>(w) & 15) != 0) return FERRITE_DECLINED;
+    if (x_dtype == FERRITE_DT_F32)
+        matmul_exact_kernel<float><<<grid, 256, 0, st>>>((const float*)x, w, bias, out, n, k, o);
+    else if (x_dtype == FERRITE_DT_BF16)
+        matmul_exact_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)x, w, bias, out, n, k, o);
+    else
+        return FERRITE_ERR_INVALID_ARG;
+    return check_launch("matmul_exact");
+}
+
+// Any-k variant: one lane per output straight from global memory (small or unaligned problems).
+__global__ void matmul_exact_simple_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                           const float* __restrict__ bias, float* __restrict__ out, int n, int k,
+                                           int o) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)n * o) return;
+    int t = (int)(idx / o), j = (int)(idx % o);
+    float s = 0.0f;
+    for (int l = 0; l < k; ++l) s = fadd(s, fmul(x[(size_t)t * k + l], w[(size_t)j * k + l]));
+    if (bias) s = fadd(s, bias[j]);
+    out[idx] = s;
+}
+
+// ------------------------------------------------------------------------------------------------
+// clamped SwiGLU (cpu.rs:178-203)
+// ------------------------------------------------------------------------------------------------
+__global__ void swiglu_kernel(const float* __restrict__ gate_up, float limit, float* __restrict__ out, int n,
+                              int inter) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)n * inter) return;
+    size_t i = idx / inter, j = idx % inter;
+    out[idx] = swiglu_ref(gate_up[i * 2 * inter + j], gate_up[i * 2 * inter + inter + j], limit);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Routing: one wave per token.  sigmoid -> +bias -> (group top-2 sums -> keep topk_group groups) ->
+// k rounds of wave-wide arg-max on (choice, lower index wins) -> renormalised weights from the raw sigmoid.
+// Semantics and operation order follow cpu.rs:546-569; ties -> lower index (cpu.rs:560).
+// ------------------------------------------------------------------------------------------------
+constexpr int RT_MAX_E = 512;
+constexpr int RT_NI = RT_MAX_E / 64;
+constexpr int RT_MAX_K = 32;
+
+__device__ __forceinline__ uint32_t ordered_u32(float f) {
+    uint32_t u = f2u(f);
+    return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        unsigned long long o = __shfl_xor(v, off, 64);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
+                                                        const float* __restrict__ bias, int n, int e, int topk,
+                                                        int n_group, int topk_group, float scaling,
+                                                        float* __restrict__ probs, float* __restrict__ ids_f32,
+                                                        int32_t* __restrict__ ids_i32) {
+    __shared__ float choice_lds[4][RT_MAX_E];
+    __shared__ uint8_t keep_lds[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    const bool live = t < n;
+    const int ni = (e + 63) >> 6;
+
+    float sg[RT_NI], ch[RT_NI];
+    bool ok[RT_NI];
+#pragma unroll
+    for (int i = 0; i < RT_NI; ++i) {
+        int j = lane + 64 * i;
+        ok[i] = live && i < ni && j < e;
+        float l = ok[i] ? logits[(size_t)t * e + j] : 0.0f;
+        sg[i] = sigmoid_ref(l);
+        ch[i] = ok[i] ? fadd(sg[i], bias ? bias[j] : 0.0f) : 0.0f;
+    }
+
+    if (n_group > 1) {
+        const int gs = e / n_group;
+#pragma unroll
+        for (int i = 0; i < RT_NI; ++i) {
+            int j = lane + 64 * i;
+            if (i < ni && j < e) choice_lds[wave][j] = ch[i];
+        }
+        __syncthreads();
+        // lane g scores group g: largest + second largest choice (largest first)
+        float gscore = 0.0f;
+        if (lane < n_group) {
+            float m1 = u2f(0xff800000u), m2 = u2f(0xff800000u);
+            for (int j = lane * gs; j < (lane + 1) * gs; ++j) {
+                float c = choice_lds[wave][j];
+                if (c > m1) { m2 = m1; m1 = c; }
+                else if (c > m2) m2 = c;
+            }
+            gscore = gs > 1 ? fadd(m1, m2) : m1;
+        }
+        // rank of group g under (score desc, index asc)
+        int rank = 0;
+        for (int g2 = 0; g2 < n_group; ++g2) {
+            float s2 = __shfl(gscore, g2, 64);
+            rank += (s2 > gscore || (s2 == gscore && g2 < lane)) ? 1 : 0;
+        }
+        if (lane < n_group) keep_lds[wave][lane] = rank < topk_group ? 1 : 0;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < RT_NI; ++i) {
+            int j = lane + 64 * i;
+            if (ok[i] && !keep_lds[wave][j / gs]) ok[i] = false;
+        }
+    }
+
+    unsigned long long key[RT_NI];
+#pragma unroll
+    for (int i = 0; i < RT_NI; ++i) {
+        uint32_t j = lane + 64 * i;
+        key[i] = ok[i] ? (((unsigned long long)ordered_u32(ch[i]) << 32) | (0xFFFFFFFFu - j)) : 0ull;
+    }
+
+    int my_id = -1;
+    float my_sig = 0.0f;
+    for (int r = 0; r < topk; ++r) {
+        unsigned long long best = 0ull;
+#pragma unroll
+        for (int i = 0; i < RT_NI; ++i) best = key[i] > best ? key[i] : best;
+        best = wave_max_u64(best);
+        uint32_t j = 0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFull);
+        int wi = (int)(j >> 6), wl = (int)(j & 63);
+        float sv = 0.0f;
+#pragma unroll
+        for (int i = 0; i < RT_NI; ++i) {
+            if (i == wi) {
+                sv = sg[i];
+                if (lane == wl) key[i] = 0ull;
+            }
+        }
+        sv = __shfl(sv, wl, 64);
+        if (lane == r) {
+            my_id = best ? (int)j : -1;
+            my_sig = sv;
+        }
+    }
+    // cpu.rs:562-568: sum in selection order, then sig / (sum + f32::EPSILON) * scale
+    float sum = 0.0f;
+    for (int r = 0; r < topk; ++r) sum = fadd(sum, __shfl(my_sig, r, 64));
+    if (live && lane < topk) {
+        size_t o = (size_t)t * topk + lane;
+        probs[o] = fmul(fdiv(my_sig, fadd(sum, 1.1920928955078125e-07f)), scaling);
+        if (ids_f32) ids_f32[o] = (float)my_id;
+        if (ids_i32) ids_i32[o] = my_id;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stable permutation by expert.  Every token holds each expert at most once, so the assignments of expert e
+// in ascending flat index are its tokens in ascending order: rank = number of earlier tokens that chose e.
+// Tokens are cut into chunks of 64 (one wave); per (expert, chunk) a 64-bit membership mask is built with
+// LDS atomics; a per-expert prefix over chunks plus a popcount below the token's bit gives the rank, and an
+// exclusive scan of the per-expert totals gives the expert's first grouped row.  No global atomics and no
+// dependence on scheduling: the tables are a pure function of ids.
+//   phase A: masks    phase B: per-expert chunk prefixes, expert scan, active list, unit tables
+//   phase C: scatter
+// n <= 1024 runs A,B,C in one block with the masks in LDS; larger n uses three launches with the masks in
+// the caller's scratch.
+// ------------------------------------------------------------------------------------------------
+constexpr int PM_MAX_E = 512;
+constexpr int PM_SMALL_N = 1024;
+
+struct PermArgs {
+    const int32_t* ids;
+    int n, topk, n_experts;
+    int32_t *counts, *starts, *perm_map, *gather_src, *active, *n_active;
+    int32_t *unit_expert, *unit_row0, *unit_rows, *n_units;
+    int unit_cap, max_units, has_shared;
+};
+
+// wave 0 of a block: exclusive scan over experts + active list + unit tables. cnt[] readable by the wave.
+__device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t* starts_lds) {
+    const int lane = threadIdx.x & 63;
+    const int E = a.n_experts;
+    const int per = (E + 63) >> 6;            // experts per lane (<= 8)
+    const int e0 = lane * per;
+    int tot = 0, nact = 0, ntile = 0;
+    for (int i = 0; i < per; ++i) {
+        int e = e0 + i;
+        if (e < E) {
+            int c = cnt[e];
+            tot += c;
+            nact += c > 0;
+            if (a.unit_cap > 0) ntile += (c + a.unit_cap - 1) / a.unit_cap;
+        }
+    }
+    // inclusive wave scans
+    int s_tot = tot, s_act = nact, s_tile = ntile;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        int v0 = __shfl_up(s_tot, off, 64), v1 = __shfl_up(s_act, off, 64), v2 = __shfl_up(s_tile, off, 64);
+        if (lane >= off) { s_tot += v0; s_act += v1; s_tile += v2; }
+    }
+    int run = s_tot - tot, ract = s_act - nact, rtile = s_tile - ntile;
+    const int total = __shfl(s_tot, 63, 64), total_act = __shfl(s_act, 63, 64), total_tile = __shfl(s_tile, 63, 64);
+    for (int i = 0; i < per; ++i) {
+        int e = e0 + i;
+        if (e < E) {
+            int c = cnt[e];
+            a.counts[e] = c;
+            a.starts[e] = run;
+            starts_lds[e] = run;
+            if (c > 0 && a.active) a.active[ract] = e;
+            ract += c > 0;
+            if (a.unit_cap > 0) {
+                for (int r = 0; r < c; r += a.unit_cap) {
+                    if (rtile < a.max_units) {
+                        a.unit_expert[rtile] = e;
+                        a.unit_row0[rtile] = run + r;
+                        a.unit_rows[rtile] = min(a.unit_cap, c - r);
+                    }
+                    ++rtile;
+                }
+            }
+            run += c;
+        }
+    }
+    if (lane == 0) {
+        a.starts[E] = total;
+        starts_lds[E] = total;
+        if (a.n_active) *a.n_active = total_act;
+    }
+    if (a.active)
+        for (int i = total_act + lane; i < E; i += 64) a.active[i] = -1;
+    if (a.unit_cap > 0) {
+        // shared expert: all n tokens, rows [n*topk, n*topk + n) of the activation / output row space
+        int sh_tiles = a.has_shared ? (a.n + a.unit_cap - 1) / a.unit_cap : 0;
+        for (int i = lane; i < sh_tiles; i += 64) {
+            int u = total_tile + i;
+            if (u < a.max_units) {
+                a.unit_expert[u] = E;
+                a.unit_row0[u] = a.n * a.topk + i * a.unit_cap;
+                a.unit_rows[u] = min(a.unit_cap, a.n - i * a.unit_cap);
+            }
+        }
+        if (lane == 0) *a.n_units = min(total_tile + sh_tiles, a.max_units);
+    }
+}
+
+__global__ __launch_bounds__(1024) void permute_small_kernel(PermArgs a) {
+    extern __shared__ unsigned long long pm_lds[];
+    const int E = a.n_experts, n = a.n, k = a.topk;
+    const int nchunk = (n + 63) >> 6;
+    unsigned long long* mask = pm_lds;                                   // [E][nchunk]
+    int32_t* offs = reinterpret_cast<int32_t*>(mask + (size_t)E * nchunk);  // [E][nchunk]
+    int32_t* cnt = offs + (size_t)E * nchunk;                            // [E]
+    int32_t* starts_lds = cnt + E;                                       // [E+1]
+    const int tid = threadIdx.x;
+    for (int i = tid; i < E * nchunk; i += blockDim.x) mask[i] = 0ull;
+    __syncthreads();
+    for (int t = tid; t < n; t += blockDim.x)
+        for (int j = 0; j < k; ++j) {
+            int e = a.ids[(size_t)t * k + j];
+            if (e >= 0 && e < E) atomicOr(&mask[(size_t)e * nchunk + (t >> 6)], 1ull << (t & 63));
+        }
+    __syncthreads();
+    for (int e = tid; e < E; e += blockDim.x) {
+        int run = 0;
+        for (int c = 0; c < nchunk; ++c) {
+            offs[(size_t)e * nchunk + c] = run;
+            run += __popcll(mask[(size_t)e * nchunk + c]);
+        }
+        cnt[e] = run;
+    }
+    __syncthreads();
+    if (tid < 64) perm_expert_scan(a, cnt, starts_lds);
+    __syncthreads();
+    const int total = starts_lds[E];
+    for (int t = tid; t < n; t += blockDim.x)
+        for (int j = 0; j < k; ++j) {
+            int i = t * k + j;
+            int e = a.ids[i];
+            if (e < 0 || e >= E) { a.perm_map[i] = -1; continue; }
+            unsigned long long m = mask[(size_t)e * nchunk + (t >> 6)];
+            int g = starts_lds[e] + offs[(size_t)e * nchunk + (t >> 6)] + __popcll(m & ((1ull << (t & 63)) - 1ull));
+            a.perm_map[i] = g;
+            a.gather_src[g] = i;
+        }
+    for (int g = total + tid; g < n * k; g += blockDim.x) a.gather_src[g] = -1;
+}
+
+// large-n phase A: one wave per 64-token chunk
+__global__ __launch_bounds__(256) void permute_mask_kernel(PermArgs a, unsigned long long* __restrict__ gmask) {
+    extern __shared__ unsigned long long pm_lds[];
+    const int E = a.n_experts, n = a.n, k = a.topk;
+    const int nchunk = (n + 63) >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int chunk = blockIdx.x * 4 + wave;
+    unsigned long long* m = pm_lds + (size_t)wave * E;
+    for (int e = lane; e < E; e += 64) m[e] = 0ull;
+    __syncthreads();
+    int t = chunk * 64 + lane;
+    if (chunk < nchunk && t < n)
+        for (int j = 0; j < k; ++j) {
+            int e = a.ids[(size_t)t * k + j];
+            if (e >= 0 && e < E) atomicOr(&m[e], 1ull << lane);
+        }
+    __syncthreads();
+    if (chunk < nchunk)
+        for (int e = lane; e < E; e += 64) gmask[(size_t)e * nchunk + chunk] = m[e];
+}
+
+// large-n phase B: one block; thread e walks its chunks
+__global__ __launch_bounds__(512) void permute_scan_kernel(PermArgs a, const unsigned long long* __restrict__ gmask,
+                                                           int32_t* __restrict__ goffs) {
+    __shared__ int32_t cnt[PM_MAX_E];
+    __shared__ int32_t starts_lds[PM_MAX_E + 1];
+    const int E = a.n_experts;
+    const int nchunk = (a.n + 63) >> 6;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int run = 0;
+        for (int c = 0; c < nchunk; ++c) {
+            goffs[(size_t)e * nchunk + c] = run;
+            run += __popcll(gmask[(size_t)e * nchunk + c]);
+        }
+        cnt[e] = run;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) perm_expert_scan(a, cnt, starts_lds);
+}
+
+// large-n phase C
+__global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const unsigned long long* __restrict__ gmask,
+                                                              const int32_t* __restrict__ goffs) {
+    const int E = a.n_experts, n = a.n, k = a.topk;
+    const int nchunk = (n + 63) >> 6;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)n * k) return;
+    const int total = a.starts[E];
+    if ((int)i >= total) a.gather_src[i] = -1;   // positions no assignment reaches (distinct from any g below)
+    int t = (int)(i / k);
+    int e = a.ids[i];
+    if (e < 0 || e >= E) { a.perm_map[i] = -1; return; }
+    unsigned long long m = gmask[(size_t)e * nchunk + (t >> 6)];
+    int g = a.starts[e] + goffs[(size_t)e * nchunk + (t >> 6)] + __popcll(m & ((1ull << (t & 63)) - 1ull));
+    a.perm_map[i] = g;
+    a.gather_src[g] = (int)i;
+}
+
+static size_t perm_scratch_bytes(int n, int n_experts) {
+    size_t nchunk = ((size_t)n + 63) / 64;
+    return (size_t)n_experts * nchunk * (8 + 4) + 64;
+}
+
+int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* counts, int32_t* starts,
+                   int32_t* perm_map, int32_t* gather_src, int32_t* active, int32_t* n_active, void* scratch,
+                   size_t scratch_bytes, const UnitTables* units, int has_shared, hipStream_t st) {
+    if (n <= 0 || topk <= 0 || n_experts <= 0 || n_experts > PM_MAX_E) return FERRITE_ERR_INVALID_ARG;
+    PermArgs a{};
+    a.ids = ids; a.n = n; a.topk = topk; a.n_experts = n_experts;
+    a.counts = counts; a.starts = starts; a.perm_map = perm_map; a.gather_src = gather_src;
+    a.active = active; a.n_active = n_active; a.has_shared = has_shared;
+    if (units) {
+        a.unit_expert = units->unit_expert; a.unit_row0 = units->unit_row0; a.unit_rows = units->unit_rows;
+        a.n_units = units->n_units; a.unit_cap = units->unit_rows_cap; a.max_units = units->max_units;
+    }
+    const int nchunk = (n + 63) / 64;
+    const size_t lds = (size_t)n_experts * nchunk * 12 + (size_t)(2 * n_experts + 1) * 4;
+    if (n <= PM_SMALL_N && lds <= 60 * 1024) {
+        permute_small_kernel<<<1, 1024, lds, st>>>(a);
+        return check_launch("permute_small");
+    }
+    if (scratch == nullptr || scratch_bytes < perm_scratch_bytes(n, n_experts)) return FERRITE_ERR_WORKSPACE;
+    unsigned long long* gmask = reinterpret_cast<unsigned long long*>(scratch);
+    int32_t* goffs = reinterpret_cast<int32_t*>(gmask + (size_t)n_experts * nchunk);
+    permute_mask_kernel<<<(nchunk + 3) / 4, 256, (size_t)4 * n_experts * 8, st>>>(a, gmask);
+    int rc = check_launch("permute_mask");
+    if (rc) return rc;
+    permute_scan_kernel<<<1, 512, 0, st>>>(a, gmask, goffs);
+    rc = check_launch("permute_scan");
+    if (rc) return rc;
+    size_t na = (size_t)n * topk;
+    permute_scatter_kernel<<<(unsigned)((na + 255) / 256), 256, 0, st>>>(a, gmask, goffs);
+    return check_launch("permute_scatter");
+}
+
+}  // namespace fe
+
+using namespace fe;
+
+extern "C" int ferrite_matmul_f32(const float* x, const float* w, const float* bias, float* out, int n, int k,
+                                  int o, ferrite_stream_t stream) {
+    if (n < 0 || k < 0 || o < 0) return FERRITE_ERR_INVALID_ARG;
+    if (n == 0 || o == 0) return FERRITE_OK;
+    if ((n > 0 && !x) || !w || !out) return FERRITE_ERR_INVALID_ARG;
+    hipStream_t st = as_stream(stream);
+    if ((k & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0 && (size_t)n * o >= 1024)
+        return launch_matmul_exact(x, FERRITE_DT_F32, w, bias, out, n, k, o, st);
+    size_t total = (size_t)n * o;
+    matmul_exact_simple_kernel<<<(unsigned)((total + 63) / 64), 64, 0, st>>>(x, w, bias, out, n, k, o);
+    return check_launch("matmul_exact_simple");
+}
+
+extern "C" int ferrite_swiglu_limited_f32(const float* gate_up, float limit, float* out, int n, int inter,
+                                          ferrite_stream_t stream) {
+    if (n < 0 || inter < 0) return FERRITE_ERR_INVALID_ARG;
+    size_t total = (size_t)n * inter;
+    if (total == 0) return FERRITE_OK;
+    if (!gate_up || !out) return FERRITE_ERR_INVALID_ARG;
+    swiglu_kernel<<<(unsigned)((total + 255) / 256), 256, 0, as_stream(stream)>>>(gate_up, limit, out, n, inter);
+    return check_launch("swiglu");
+}
+
+extern "C" int ferrite_moe_route(const float* logits, const float* bias, int n, int e, int topk, int n_group,
+                                 int topk_group, float routed_scaling, float* probs, float* ids_f32,
+                                 int32_t* ids_i32, ferrite_stream_t stream) {
+    if (n < 0 || e <= 0 || topk <= 0 || topk > e || !logits || !probs) return FERRITE_ERR_INVALID_ARG;
+    if (n_group < 1) n_group = 1;
+    if (n_group > 1) {
+        if (e % n_group != 0 || topk_group < 1 || topk_group > n_group) return FERRITE_ERR_INVALID_ARG;
+        if (topk > topk_group * (e / n_group)) return FERRITE_ERR_INVALID_ARG;
+        if (n_group > 64) return FERRITE_DECLINED;
+        if (topk_group == n_group) n_group = 1;  // keeps every expert: the ungrouped router
+    }
+    if (e > RT_MAX_E || topk > RT_MAX_K) return FERRITE_DECLINED;
+    if (n == 0) return FERRITE_OK;
+    moe_route_kernel<<<(n + 3) / 4, 256, 0, as_stream(stream)>>>(logits, bias, n, e, topk, n_group, topk_group,
+                                                                 routed_scaling, probs, ids_f32, ids_i32);
+    return check_launch("moe_route");
+}
+
+extern "C" size_t ferrite_moe_permute_scratch_bytes(int n, int n_experts) {
+    if (n <= 0 || n_experts <= 0) return 0;
+    return perm_scratch_bytes(n, n_experts);
+}
+
+extern "C" int ferrite_moe_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* counts,
+                                   int32_t* starts, int32_t* perm_map, int32_t* gather_src, int32_t* active,
+                                   int32_t* n_active, void* scratch, size_t scratch_bytes,
+                                   ferrite_stream_t stream) {
+    if (!ids || !counts || !starts || !perm_map || !gather_src) return FERRITE_ERR_INVALID_ARG;
+    return launch_permute(ids, n, topk, n_experts, counts, starts, perm_map, gather_src, active, n_active, scratch,
+                          scratch_bytes, nullptr, 0, as_stream(stream));
+}

@@ -1,0 +1,165 @@
+/*
+ * ferrite_hip.h -- C ABI of libferrite_hip.so: the MoE FFN layer of ferrite on one MI355X (gfx950).
+ *
+ * This is what a `HipBackend` in crates/ferrite-kernel would bind through dlopen, in the same way the
+ * reference's CudaBackend binds libferrite_kernels.so (crates/ferrite-kernel/src/cuda.rs:24-400,5339-5427).
+ * Conventions, all taken from that boundary:
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - entry points return 0 on success and a non-zero FERRITE_* code otherwise (cuda.rs:411-425 maps
+ *     non-zero to FerriteError::InvalidArg); FERRITE_DECLINED means "this shape is outside the kernel's
+ *     contract, use another path" (kernels/cuda/dsv41_moe_align.cu:50-52);
+ *   - launchers never allocate, never synchronise and never read the environment, so any of them may be
+ *     recorded into a stream capture (cuda.rs:3008-3011); all scratch memory comes from the caller;
+ *   - matrices are row-major, weights are [out_features, in_features] and ops compute x . w^T
+ *     (crates/ferrite-kernel/src/lib.rs:61-66);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ */
+#ifndef FERRITE_HIP_H
+#define FERRITE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FERRITE_OK 0
+#define FERRITE_ERR_INVALID_ARG 1  /* FerriteError::InvalidArg / ShapeMismatch */
+#define FERRITE_DECLINED 2         /* shape outside this kernel's contract */
+#define FERRITE_ERR_WORKSPACE 3    /* workspace too small */
+#define FERRITE_ERR_RUNTIME 4      /* a HIP runtime call failed: see ferrite_hip_last_error() */
+
+#define FERRITE_ABI_VERSION 1u
+
+/* dtype tags for activation buffers (ferrite-types DType, crates/ferrite-types/src/lib.rs:16-25) */
+#define FERRITE_DT_F32 0
+#define FERRITE_DT_BF16 1
+
+/* layer arithmetic modes */
+#define FERRITE_MODE_F32_CHECK 0   /* f32 activations, weights dequantised exactly, f32 FMA dot products */
+#define FERRITE_MODE_MFMA_FP8 1    /* activations quantised e4m3 per 32 (e8m0 scale), block-scaled MFMA */
+
+typedef void* ferrite_stream_t;
+
+/* ---- identity: ferrite_kernels.cu:50-52, checked right after dlopen (cuda.rs:2061-2102) ---- */
+const char* ferrite_kernel_build_id(void);
+unsigned ferrite_kernel_abi_version(void);
+/* Text of the last HIP runtime error seen by this thread ("" if none). */
+const char* ferrite_hip_last_error(void);
+
+/* ---- KernelBackend ops on the path (f32 device buffers, like the reference's GLM ABI) ---- */
+
+/* KernelBackend::matmul (lib.rs:73; cpu.rs:82-122): out[n,o] = x[n,k] . w[o,k]^T (+ bias[o], may be NULL).
+ * Each output is the reference's sequential-k f32 chain (separate multiply and add), bit for bit. */
+int ferrite_matmul_f32(const float* x, const float* w, const float* bias, float* out, int n, int k, int o,
+                       ferrite_stream_t stream);
+
+/* KernelBackend::swiglu_limited (lib.rs:83-85; cpu.rs:178-203): gate_up [n, 2*inter] gate first. */
+int ferrite_swiglu_limited_f32(const float* gate_up, float limit, float* out, int n, int inter,
+                               ferrite_stream_t stream);
+
+/* KernelBackend::moe_route (lib.rs:194-206; cpu.rs:528-572) extended with group-limited selection
+ * (n_group = 1 is the reference's router).  probs [n,topk]; ids_f32 [n,topk] (the reference ABI stores ids
+ * as f32) and/or ids_i32 [n,topk]; either ids pointer may be NULL.  Requires e <= 512, topk <= 32,
+ * e % n_group == 0, topk <= topk_group * e / n_group. */
+int ferrite_moe_route(const float* logits, const float* bias, int n, int e, int topk, int n_group,
+                      int topk_group, float routed_scaling, float* probs, float* ids_f32, int32_t* ids_i32,
+                      ferrite_stream_t stream);
+
+/* Token permutation by expert (kernels/cuda/dsv41_route.cu:194-315 contract; host golden
+ * crates/ferrite-models/src/dsv41/chain_dev.rs:862-899): grouped order = expert ascending, then flat
+ * assignment index i = t*topk + j ascending.  ids [n,topk] i32 with distinct experts per token; ids outside
+ * [0, n_experts) drop out (perm_map = -1).  Outputs: counts[E], starts[E+1], perm_map[n*topk] (original ->
+ * grouped), gather_src[n*topk] (grouped -> original, -1 past the end), active[E] (ascending experts with
+ * counts > 0, -1 padded), n_active[1].  scratch: ferrite_moe_permute_scratch_bytes(n, n_experts) bytes. */
+size_t ferrite_moe_permute_scratch_bytes(int n, int n_experts);
+int ferrite_moe_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* counts, int32_t* starts,
+                        int32_t* perm_map, int32_t* gather_src, int32_t* active, int32_t* n_active,
+                        void* scratch, size_t scratch_bytes, ferrite_stream_t stream);
+
+/* MXFP4 -> f32 (crates/ferrite-models/src/dsv41/quant.rs:260-278): w [rows, cols/2] u8 (low nibble = even
+ * column), scale [rows, cols/32] e8m0 -> dst [rows, cols] f32, exact. */
+int ferrite_mxfp4_dequant(const uint8_t* w, const uint8_t* scale, int64_t rows, int64_t cols, float* dst,
+                          ferrite_stream_t stream);
+
+/* Activation quantisation (quant.rs:190-214, block 32, power-of-two scale): x [rows, cols] (f32 or bf16) ->
+ * q [rows, cols] e4m3 codes, scale [rows, cols/32] e8m0 bytes (2^(b-127)). */
+int ferrite_act_quant_fp8(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale,
+                          ferrite_stream_t stream);
+
+/* ---- the fused layer: the counterpart of CudaBackend::moe_layer_dev (cuda.rs:5604-6142) for MXFP4 experts
+ *      with group-limited routing; caller = Engine::moe_ffn (crates/ferrite-exec/src/lib.rs:1083-1166) ---- */
+
+typedef struct ferrite_moe_shape {
+    int hidden;        /* H, multiple of 128 */
+    int n_experts;     /* E routed experts */
+    int topk;          /* k */
+    int inter;         /* I  = moe_intermediate, multiple of 128 */
+    int shared_inter;  /* Is = shared expert intermediate (0 = none), multiple of 128 */
+    int n_group;       /* 1 = ungrouped */
+    int topk_group;
+    float routed_scaling;
+    float swiglu_limit;
+} ferrite_moe_shape;
+
+/* Checkpoint-layout MXFP4 weights (crates/ferrite-models/src/dsv41/weights.rs:340-341): codes
+ * [E, rows, cols/2] u8 and e8m0 scales [E, rows, cols/32] u8, experts stacked contiguously. */
+typedef struct ferrite_moe_weights {
+    const float* router_w;     /* [E, H] f32 */
+    const float* router_bias;  /* [E] f32 or NULL (zeros) */
+    const uint8_t *gate_w, *gate_s; /* [E, I, H/2], [E, I, H/32] */
+    const uint8_t *up_w, *up_s;
+    const uint8_t *down_w, *down_s; /* [E, H, I/2], [E, H, I/32] */
+    const uint8_t *sh_gate_w, *sh_gate_s, *sh_up_w, *sh_up_s; /* [Is, H/2], [Is, H/32] */
+    const uint8_t *sh_down_w, *sh_down_s;                     /* [H, Is/2], [H, Is/32] */
+} ferrite_moe_weights;
+
+/* One-time repack of the checkpoint layout into the tile order the MFMA kernels stream (a pure permutation
+ * of bytes; the reference does the analogous gate/up interleave at load time,
+ * kernels/cuda/dsv41_experts_mxf4.cu:3430).  `packed` must hold ferrite_moe_packed_bytes(shape) bytes. */
+size_t ferrite_moe_packed_bytes(const ferrite_moe_shape* shape);
+int ferrite_moe_pack_weights(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, uint8_t* packed,
+                             ferrite_stream_t stream);
+/* Inverse view for verification: dequantise matrix `which` (0 gate, 1 up, 2 down) of expert `expert`
+ * (expert == n_experts selects the shared expert) from the packed buffer to f32 [rows, cols]. */
+int ferrite_moe_packed_dequant(const ferrite_moe_shape* shape, const uint8_t* packed, int expert, int which,
+                               float* dst, ferrite_stream_t stream);
+
+/* Pointers into the caller's workspace where the layer leaves its intermediates (for tests / tracing). */
+typedef struct ferrite_moe_workspace_view {
+    float* logits;       /* [n, E] */
+    float* probs;        /* [n, topk] */
+    float* ids_f32;      /* [n, topk] */
+    int32_t* ids;        /* [n, topk] */
+    int32_t* counts;     /* [E] */
+    int32_t* starts;     /* [E+1] */
+    int32_t* perm_map;   /* [n*topk] */
+    int32_t* gather_src; /* [n*topk] */
+    int32_t* active;     /* [E] */
+    int32_t* n_active;   /* [1] */
+    float* y;            /* [(n*topk + n), H] expert outputs in grouped order, then the shared expert's rows */
+} ferrite_moe_workspace_view;
+
+size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
+int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int mode, void* workspace,
+                                     ferrite_moe_workspace_view* view_host);
+
+/* The layer.  x [n, H] (x_dtype), out [n, H] (out_dtype).  mode FERRITE_MODE_F32_CHECK reads `w` (checkpoint
+ * layout) and requires f32 x; FERRITE_MODE_MFMA_FP8 reads `packed` (+ w->router_w / router_bias).
+ * The launch sequence depends only on (shape, n, mode), never on the routing, so a captured graph of it
+ * replays correctly for any input (the GraphCapable contract, crates/ferrite-kernel/src/graph.rs:48-64). */
+int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, const uint8_t* packed,
+                            const void* x, int x_dtype, int n, void* out, int out_dtype, int mode,
+                            void* workspace, size_t workspace_bytes, ferrite_stream_t stream);
+
+/* ---- graph capture: ferrite_graph_begin/end/instantiate/launch (cuda.rs:284-287) ---- */
+int ferrite_graph_begin(ferrite_stream_t stream);
+int ferrite_graph_end(ferrite_stream_t stream, void** graph_exec_out);
+int ferrite_graph_launch(void* graph_exec, ferrite_stream_t stream);
+int ferrite_graph_destroy(void* graph_exec);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

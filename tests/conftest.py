@@ -18,3 +18,10 @@ def oracle():
     from oracle import binding
     binding.build()
     return binding
+
+
+@pytest.fixture(scope="session")
+def hip():
+    """The HIP backend over libferrite_hip.so (GPU tests only; it has no CPU path)."""
+    from ferrite_amd.backend import HipBackend
+    return HipBackend()

@@ -1,0 +1,135 @@
+"""GPU parity of the fused MoE layer against the CPU oracle (and the committed golden vectors).
+
+Bars: router ids, probs' inputs, permutation tables: bit-exact.  Layer output: max|d|/max|ref| <= 1e-5 in the
+f32 check mode; <= 2e-2 in the MFMA mode against the oracle evaluated with the same e4m3-per-32 activation
+quantisation (crates/ferrite-models/src/dsv41/quant.rs:201-214)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from ferrite_amd import synth
+from ferrite_amd.backend import MODE_F32_CHECK, MODE_MFMA_FP8
+from tests.refmath import max_abs_rel
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 1e-5
+TOL_MFMA = 2e-2
+
+
+def run_layer(hip, layer, x_np, mode, bf16=False):
+    cfg = layer.cfg
+    x = torch.from_numpy(x_np).to(hip.device)
+    if bf16:
+        x = x.to(torch.bfloat16)
+    out = torch.empty(x.shape[0], cfg.hidden, dtype=torch.float32, device=hip.device)
+    hip.moe_layer_dev_mxfp4(layer, x, out, mode)
+    hip.sync()
+    v = {k: t.cpu().numpy() for k, t in hip.workspace_view(layer, x.shape[0], mode).items()}
+    return out.cpu().numpy(), v
+
+
+def check_routing(v, ref, oracle, cfg):
+    assert np.array_equal(v["logits"], ref["logits"])            # sequential-k chain, bit for bit
+    assert np.array_equal(v["ids"], ref["ids"].astype(np.int32))
+    assert np.array_equal(v["ids_f32"], ref["ids"])
+    assert np.array_equal(v["probs"], ref["probs"])
+    t = oracle.moe_permute(v["ids"], cfg.n_experts)
+    for k in ("counts", "starts", "perm_map", "gather_src", "active"):
+        assert np.array_equal(v[k], t[k]), k
+    assert int(v["n_active"][0]) == t["n_active"]
+
+
+def test_layer_c0_f32_check_mode(hip, oracle):
+    inp = synth.make_inputs(synth.CONFIGS["c0"], seed=0)
+    layer = hip.load_moe_layer(inp)
+    out, v = run_layer(hip, layer, inp.x, MODE_F32_CHECK)
+    ref = oracle.moe_ffn_mxfp4(inp)
+    check_routing(v, ref, oracle, inp.cfg)
+    assert max_abs_rel(out, ref["out"]) <= TOL_F32
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "c0_layer.npz"))
+    assert np.array_equal(v["ids"], g["ids"]) and np.array_equal(v["perm_map"], g["perm_map"])
+    assert max_abs_rel(out, g["out_f32"]) <= TOL_F32
+
+
+def test_layer_c0_mfma_mode(hip, oracle):
+    inp = synth.make_inputs(synth.CONFIGS["c0"], seed=0)
+    layer = hip.load_moe_layer(inp)
+    out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    ref = oracle.moe_ffn_mxfp4(inp, act_mode=1)
+    check_routing(v, ref, oracle, inp.cfg)
+    assert max_abs_rel(out, ref["out"]) <= TOL_MFMA
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "c0_layer.npz"))
+    assert max_abs_rel(out, g["out_fp8act"]) <= TOL_MFMA
+
+
+def test_layer_smoke_fixture(hip, oracle):
+    """crates/ferrite-kernel/tests/gpu_smoke.rs:437-562 (n=1, H 64 is below the MFMA tile: f32 mode only)."""
+    from tests.test_oracle_layer import smoke_fixture
+    inp, _ = smoke_fixture()
+    layer = hip.load_moe_layer(inp, pack=False)
+    out, v = run_layer(hip, layer, inp.x, MODE_F32_CHECK)
+    ref = oracle.moe_ffn_mxfp4(inp)
+    assert np.array_equal(v["ids"], ref["ids"].astype(np.int32))
+    assert np.abs(out - ref["out"]).max() < 1e-4       # the reference test's own tolerance (gpu_smoke.rs:566)
+
+
+@pytest.mark.parametrize("seed,n", [(1, 1), (2, 3), (3, 17), (4, 40)])
+def test_layer_small_shapes_both_modes(hip, oracle, seed, n):
+    """Ragged token counts: units of 1..16 rows, more than one unit per expert, experts with no tokens."""
+    cfg = synth.MoeConfig(n, 256, 8, 3, 256, 128, 4, 2)
+    inp = synth.make_inputs(cfg, seed=seed)
+    layer = hip.load_moe_layer(inp)
+    ref32 = oracle.moe_ffn_mxfp4(inp)
+    out, v = run_layer(hip, layer, inp.x, MODE_F32_CHECK)
+    check_routing(v, ref32, oracle, cfg)
+    assert max_abs_rel(out, ref32["out"]) <= TOL_F32
+    out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    check_routing(v, ref32, oracle, cfg)
+    assert max_abs_rel(out, oracle.moe_ffn_mxfp4(inp, act_mode=1)["out"]) <= TOL_MFMA
+
+
+def test_layer_c1_decode(hip, oracle):
+    """The decode benchmark shape: 32 tokens, H 4096, 128 experts, top-8 of 8 groups, I 1536, bf16 activations."""
+    inp = synth.make_inputs(synth.CONFIGS["c1"], seed=0)
+    layer = hip.load_moe_layer(inp)
+    ref32 = oracle.moe_ffn_mxfp4(inp, n_threads=16)
+    out, v = run_layer(hip, layer, inp.x, MODE_F32_CHECK)
+    check_routing(v, ref32, oracle, inp.cfg)
+    assert max_abs_rel(out, ref32["out"]) <= TOL_F32
+    out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8, bf16=True)
+    check_routing(v, ref32, oracle, inp.cfg)
+    ref8 = oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=16)
+    err = max_abs_rel(out, ref8["out"])
+    print(f"c1 mfma vs fp8-act oracle {err:.3e}; vs f32 oracle {max_abs_rel(out, ref32['out']):.3e}")
+    assert err <= TOL_MFMA
+
+
+def test_layer_graph_capture_replays(hip, oracle):
+    """GraphCapable: capture once, replay with fresh data in the same static buffers; every replay must equal the
+    eager result for that input (the launch sequence is routing independent)."""
+    cfg = synth.CONFIGS["c0"].with_tokens(24)
+    inp = synth.make_inputs(cfg, seed=7)
+    layer = hip.load_moe_layer(inp)
+    x_static = torch.zeros(24, cfg.hidden, device=hip.device)
+    out_static = torch.zeros(24, cfg.hidden, device=hip.device)
+    hip.workspace(layer, 24, MODE_MFMA_FP8)          # warm the pool before capture (cuda.rs:627-657)
+    hip.moe_layer_dev_mxfp4(layer, x_static, out_static, MODE_MFMA_FP8)
+    hip.sync()
+    hip.begin_capture()
+    hip.moe_layer_dev_mxfp4(layer, x_static, out_static, MODE_MFMA_FP8)
+    trace = hip.end_capture()
+    assert [r.op for r in trace.ops] == ["moe_layer_mxfp4"]
+    for seed in (11, 12, 13, 14):
+        x = synth.random_normal(seed, 1, 24 * cfg.hidden).reshape(24, cfg.hidden)
+        eager = torch.empty_like(out_static)
+        hip.moe_layer_dev_mxfp4(layer, torch.from_numpy(x).to(hip.device), eager, MODE_MFMA_FP8)
+        hip.sync()
+        x_static.copy_(torch.from_numpy(x))
+        torch.cuda.synchronize()
+        hip.begin_verify(trace)
+        assert hip.end_verify()
+        assert torch.equal(out_static, eager)
+    hip.graph_destroy(trace)
