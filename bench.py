@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE FFN layer on one MI355X.
+
+One "step" = one pass of the fused layer (router GEMM -> routing -> permutation -> activation quantisation ->
+gate/up GEMM + SwiGLU -> down GEMM -> combine) over one batch of synthetic tokens, replayed from a captured
+hipGraph the way a decode step runs in production.  Inputs and weights are resident in HBM before the timed
+region.  Prints ONE JSON line (see README / DESIGN for the fields).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline]
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+MFMA_PEAK_FP8_TFLOPS = 5000.0  # dense fp8-operand MFMA (e4m3 activations x e2m1 weights run at this rate)
+MFMA_PEAK_FP4_TFLOPS = 10100.0 # dense MXFP4 x MXFP4
+
+WORKLOADS = {
+    "c0": "c0: tiny parity layer, 8 tokens, H256 E16 top4 (4 groups/2) I128, MXFP4 weights, f32 activations",
+    "c1": "c1: GLM-5.3-Flash-shaped decode MoE layer, 32 tokens, H4096 E128+1 shared top8 (8 groups/4) I1536, "
+          "MXFP4 weights, bf16 activations",
+    "c2": "c2: same layer at prefill chunk, 4096 tokens, e4m3/32 activations",
+    "c4": "c4-layer: one layer of the 192-token decode step (batch 64 x MTP 3)",
+}
+
+
+class HipEvents:
+    """hipEvent_t handles through the HIP runtime (events must live on the stream the kernels run on)."""
+
+    def __init__(self):
+        self.rt = C.CDLL("libamdhip64.so")
+        self.rt.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.rt.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.rt.hipEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        self.rt.hipEventSynchronize.argtypes = [C.c_void_p]
+        self.rt.hipEventDestroy.argtypes = [C.c_void_p]
+
+    def create(self, n):
+        evs = (C.c_void_p * n)()
+        for i in range(n):
+            e = C.c_void_p()
+            if self.rt.hipEventCreate(C.byref(e)) != 0:
+                raise RuntimeError("hipEventCreate failed")
+            evs[i] = e
+        return evs
+
+    def elapsed_ms(self, a, b) -> float:
+        ms = C.c_float()
+        rc = self.rt.hipEventElapsedTime(C.byref(ms), a, b)
+        if rc != 0:
+            raise RuntimeError(f"hipEventElapsedTime rc={rc}")
+        return ms.value
+
+    def destroy(self, evs):
+        for e in evs:
+            self.rt.hipEventDestroy(e)
+
+
+def algorithmic_bytes(cfg, n, n_active):
+    """HBM bytes the layer has to move once (weights of the experts that are hit + shared, router, x, out)."""
+    H, I, Is, E = cfg.hidden, cfg.inter, cfg.shared_inter, cfg.n_experts
+    per_mat = lambda rows, cols: rows * cols // 2 + rows * cols // 32
+    gate_up = n_active * 2 * per_mat(I, H) + (2 * per_mat(Is, H) if Is else 0)
+    down = n_active * per_mat(H, I) + (per_mat(H, Is) if Is else 0)
+    router = E * H * 4
+    act = n * H * 2 * 2
+    return dict(gate_up=gate_up, down=down, router=router, act=act, total=gate_up + down + router + act)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="c1", choices=sorted(WORKLOADS))
+    ap.add_argument("--tokens", type=int, default=0, help="override the token count of the config")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of graph replays")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from ferrite_amd import synth
+    from ferrite_amd.backend import MODE_MFMA_FP8, HipBackend
+
+    cfg = synth.CONFIGS[args.config]
+    if args.tokens:
+        cfg = cfg.with_tokens(args.tokens)
+    n = cfg.n
+    hip = HipBackend()
+    t0 = time.time()
+    inp = synth.make_inputs(cfg, seed=0)
+    layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
+    t_setup = time.time() - t0
+
+    x = torch.from_numpy(inp.x).to(hip.device)
+    if cfg.act_bf16:
+        x = x.to(torch.bfloat16)
+    out = torch.empty(n, cfg.hidden, dtype=x.dtype, device=hip.device)
+    ws = hip.workspace(layer, n, MODE_MFMA_FP8)
+
+    def step():
+        hip.moe_layer_dev_mxfp4(layer, x, out, MODE_MFMA_FP8, ws)
+
+    # warm up eagerly (also raises LDS limits, fills caches), then capture one step as a graph
+    for _ in range(max(args.warmup, 2)):
+        step()
+    hip.sync()
+    trace = None
+    if not args.no_graph:
+        hip.begin_capture()
+        step()
+        trace = hip.end_capture()
+
+    def replay():
+        if trace is None:
+            step()
+        else:
+            hip.begin_verify(trace)
+
+    for _ in range(args.warmup):
+        replay()
+    hip.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        replay()
+    hip.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    # per-stage durations: eager launches with HIP events recorded on the launch stream between the stages
+    ev = HipEvents()
+    k_prof = min(args.steps, 50)
+    sets = [ev.create(8) for _ in range(k_prof)]
+    for s in sets:
+        hip.moe_layer_dev_mxfp4(layer, x, out, MODE_MFMA_FP8, ws, stage_events=s)
+    hip.sync()
+    names = ["router_gemm", "route", "permute", "act_quant", "gate_up_mfma", "down_mfma", "combine"]
+    stage_us = {nm: float(np.mean([ev.elapsed_ms(s[i], s[i + 1]) for s in sets]) * 1e3) for i, nm in enumerate(names)}
+    eager_us = float(np.mean([ev.elapsed_ms(s[0], s[7]) for s in sets]) * 1e3)
+    for s in sets:
+        ev.destroy(s)
+
+    view = hip.workspace_view(layer, n, MODE_MFMA_FP8)
+    counts = view["counts"].cpu().numpy()
+    n_active = int((counts > 0).sum())
+    ab = algorithmic_bytes(cfg, n, n_active)
+    flops = 2.0 * n * (cfg.topk * cfg.inter + cfg.shared_inter) * 3 * cfg.hidden
+
+    us_layer = ms_per_step * 1e3
+    gate_up_gbs = ab["gate_up"] / (stage_us["gate_up_mfma"] * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "kernel": "gate_up_mfma_kernel", "achieved": round(gate_up_gbs, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gate_up_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes_per_launch": ab["gate_up"], "avg_launch_us": round(stage_us["gate_up_mfma"], 2)}
+    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(traffic_file):
+        with open(traffic_file) as f:
+            roofline["traffic"] = json.load(f).get(f"gate_up_mfma_kernel:{args.config}")
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import binding as oracle
+        # the whole layer for a bounded token sample, single thread (the reference's CpuBackend is
+        # single-threaded scalar code), f32 activations as CpuBackend computes
+        ns = min(n, 32)
+        sel = np.arange(ns, dtype=np.int32)
+        reps = 0
+        t0 = time.perf_counter()
+        while True:
+            oracle.moe_ffn_mxfp4(inp, act_mode=0, n_threads=1, tok_sel=sel)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 4:
+                break
+        t1 = (time.perf_counter() - t0) / reps
+        ncores = min(16, os.cpu_count() or 1)
+        t0 = time.perf_counter()
+        oracle.moe_ffn_mxfp4(inp, act_mode=0, n_threads=ncores, tok_sel=sel)
+        tall = time.perf_counter() - t0
+        cpu = {"value": round(ns / t1, 2), "unit": "tokens/s", "cores": 1, "kind": "port",
+               "sample": f"full layer (routing of all {n} tokens + experts + shared + combine) for {ns} tokens, "
+                         f"{reps} repetition(s), {t1:.2f} s each, f32 activations",
+               "all_cores": {"value": round(ns / tall, 2), "cores": ncores, "seconds": round(tall, 2)}}
+
+    result = {
+        "metric": "moe_layer_tokens_per_s", "value": round(n / (ms_per_step * 1e-3), 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp4 x e4m3 -> f32",
+        "data": "synthetic",
+        "config": {"workload": WORKLOADS[args.config], "tokens": n, "hidden": cfg.hidden, "experts": cfg.n_experts,
+                   "topk": cfg.topk, "n_group": cfg.n_group, "topk_group": cfg.topk_group, "inter": cfg.inter,
+                   "launch": "eager" if trace is None else "hipGraph replay"},
+        "us_per_layer": round(us_layer, 2), "us_per_layer_eager_events": round(eager_us, 2),
+        "stage_us": {k: round(v, 2) for k, v in stage_us.items()},
+        "experts_hit": n_active, "max_tokens_per_expert": int(counts.max()),
+        "layer_algorithmic_bytes": ab["total"],
+        "layer_hbm_gbs": round(ab["total"] / (us_layer * 1e-6) / 1e9, 1),
+        "layer_hbm_frac": round(ab["total"] / (us_layer * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+        "layer_tflops": round(flops / (us_layer * 1e-6) / 1e12, 2),
+        "mfma_frac_of_fp8_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP8_TFLOPS, 4),
+        "mfma_frac_of_mxfp4_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP4_TFLOPS, 4),
+        "roofline": roofline, "cpu_baseline": cpu, "setup_s": round(t_setup, 1), "build_id": hip.build_id,
+    }
+    if trace is not None:
+        hip.graph_destroy(trace)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

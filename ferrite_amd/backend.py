@@ -71,7 +71,7 @@ EXPORTS = [
     "ferrite_swiglu_limited_f32", "ferrite_moe_route", "ferrite_moe_permute_scratch_bytes", "ferrite_moe_permute",
     "ferrite_mxfp4_dequant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes", "ferrite_moe_pack_weights",
     "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_workspace_view",
-    "ferrite_moe_layer_mxfp4", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
+    "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_timed", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
     "ferrite_graph_destroy",
 ]
 
@@ -100,9 +100,11 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_moe_packed_dequant.argtypes = [C.POINTER(MoeShape), vp, i32, i32, vp, vp]
     lib.ferrite_moe_layer_workspace_bytes.restype = sz
     lib.ferrite_moe_layer_workspace_bytes.argtypes = [C.POINTER(MoeShape), i32, i32]
+    lib.ferrite_moe_layer_workspace_init.argtypes = [C.POINTER(MoeShape), i32, i32, vp, sz, vp]
     lib.ferrite_moe_layer_workspace_view.argtypes = [C.POINTER(MoeShape), i32, i32, vp, C.POINTER(WorkspaceView)]
     lib.ferrite_moe_layer_mxfp4.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp, i32, i32, vp, i32,
                                             i32, vp, sz, vp]
+    lib.ferrite_moe_layer_mxfp4_timed.argtypes = lib.ferrite_moe_layer_mxfp4.argtypes + [C.POINTER(vp)]
     lib.ferrite_graph_begin.argtypes = [vp]
     lib.ferrite_graph_end.argtypes = [vp, C.POINTER(vp)]
     lib.ferrite_graph_launch.argtypes = [vp, vp]
@@ -400,11 +402,16 @@ class HipBackend:
             nbytes = self.lib.ferrite_moe_layer_workspace_bytes(C.byref(layer.shape), n, mode)
             if nbytes == 0:
                 raise InvalidArg("unsupported shape / mode")
-            layer._ws[key] = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+            self._enter()
+            self._ck(self.lib.ferrite_moe_layer_workspace_init(C.byref(layer.shape), n, mode, ws.data_ptr(), nbytes,
+                                                               self._st()), "workspace_init")
+            self._leave()
+            layer._ws[key] = ws
         return layer._ws[key]
 
     def moe_layer_dev_mxfp4(self, layer: MoeLayer, x: torch.Tensor, out: torch.Tensor, mode: int = MODE_MFMA_FP8,
-                            workspace: Optional[torch.Tensor] = None):
+                            workspace: Optional[torch.Tensor] = None, stage_events=None):
         """The whole layer on the device: router GEMM -> route -> permute -> experts -> combine (+shared).
         x [n, H] f32 or bf16, out [n, H] f32 or bf16, both pre-allocated device tensors."""
         self.recorder.record("moe_layer_mxfp4")
@@ -422,10 +429,13 @@ class HipBackend:
             raise InvalidArg("layer has no packed weights")
         ws = workspace if workspace is not None else self.workspace(layer, n, mode)
         self._enter()
-        self._ck(self.lib.ferrite_moe_layer_mxfp4(C.byref(layer.shape), C.byref(layer.weights),
-                                                  None if layer.packed is None else layer.packed.data_ptr(),
-                                                  x.data_ptr(), dts[x.dtype], n, out.data_ptr(), dts[out.dtype], mode,
-                                                  ws.data_ptr(), ws.numel(), self._st()), "moe_layer_mxfp4")
+        args = (C.byref(layer.shape), C.byref(layer.weights), None if layer.packed is None else layer.packed.data_ptr(),
+                x.data_ptr(), dts[x.dtype], n, out.data_ptr(), dts[out.dtype], mode, ws.data_ptr(), ws.numel(),
+                self._st())
+        if stage_events is None:
+            self._ck(self.lib.ferrite_moe_layer_mxfp4(*args), "moe_layer_mxfp4")
+        else:
+            self._ck(self.lib.ferrite_moe_layer_mxfp4_timed(*args, stage_events), "moe_layer_mxfp4")
 
     def workspace_view(self, layer: MoeLayer, n: int, mode: int) -> Dict[str, torch.Tensor]:
         """Typed views of the intermediates the last layer call left in its workspace."""

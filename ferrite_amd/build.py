@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 SO_PATH = os.path.join(HERE, "libferrite_hip.so")
 SOURCES = ["layer.hip", "route.hip", "formats.hip", "experts_f32.hip", "experts_mfma.hip"]
-HEADERS = ["internal.hpp", "numerics.hpp"]
+HEADERS = ["internal.hpp", "numerics.hpp", "device_utils.hpp"]
 
 
 def source_hash() -> str:

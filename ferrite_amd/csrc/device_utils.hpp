@@ -1,0 +1,51 @@
+// Device-side helpers shared by several translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "numerics.hpp"
+
+namespace fe {
+
+// act_quant_fp8 of one block of 32 consecutive values (crates/ferrite-models/src/dsv41/quant.rs:190-214,
+// power-of-two scale): 32 e4m3 codes to q (32-byte aligned) and the e8m0 scale byte as the return value.
+template <typename XT>
+__device__ __forceinline__ uint32_t quant_block32(const XT* __restrict__ src, uint8_t* __restrict__ q) {
+    float v[32];
+    if constexpr (sizeof(XT) == 4) {
+        const float4* p = reinterpret_cast<const float4*>(src);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float4 t = p[i];
+            v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+        }
+    } else {
+        const uint4* p = reinterpret_cast<const uint4*>(src);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint4 t = p[i];
+            uint32_t wds[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[8 * i + 2 * j] = u2f(wds[j] << 16);          // bf16 -> f32 is exact
+                v[8 * i + 2 * j + 1] = u2f(wds[j] & 0xffff0000u);
+            }
+        }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    const uint32_t sb = block_scale_e8m0(amax);
+    const float inv = u2f((254u - sb) << 23);   // 2^(127 - sb): exact reciprocal of the power-of-two scale
+    uint32_t out[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        out[i] = e4m3_encode(v[4 * i] * inv) | (e4m3_encode(v[4 * i + 1] * inv) << 8) |
+                 (e4m3_encode(v[4 * i + 2] * inv) << 16) | (e4m3_encode(v[4 * i + 3] * inv) << 24);
+    }
+    uint4* o = reinterpret_cast<uint4*>(q);
+    o[0] = make_uint4(out[0], out[1], out[2], out[3]);
+    o[1] = make_uint4(out[4], out[5], out[6], out[7]);
+    return sb;
+}
+
+}  // namespace fe

@@ -40,6 +40,7 @@ PackedLayout packed_layout(const ferrite_moe_shape& s) {
     L.sh_gu_scales = off; off = align_up(off + (Is / 32) * kt4(H) * 1024, 256);
     L.sh_dn_codes = off;  off = align_up(off + H * Is / 2, 256);
     L.sh_dn_scales = off; off = align_up(off + (H / 64) * kt4(Is) * 1024, 256);
+    L.router_t = off; off = align_up(off + H * ((E + 63) / 64 * 64) * 4, 256);
     L.total = off;
     return L;
 }
@@ -196,6 +197,14 @@ struct MfmaArgs {
     float limit;
 };
 
+// A unit read from device tables is used only if it is well formed.
+__device__ __forceinline__ bool unit_ok(const MfmaArgs& a, int e, int row0, int nrows) {
+    const int nk = a.n * a.topk;
+    if (nrows < 1 || nrows > 16 || row0 < 0) return false;
+    if (e == a.n_experts) return a.shared_inter > 0 && row0 >= nk && row0 + nrows <= nk + a.n;
+    return e >= 0 && e < a.n_experts && row0 + nrows <= nk;
+}
+
 // gate/up GEMM + clamped SwiGLU + e4m3-per-32 quantisation of the result.
 // grid (ceil(items / WAVES), max_units); wave w of block b owns item b*WAVES + w of the unit's expert.
 template <int WAVES>
@@ -208,6 +217,7 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
     const int u = blockIdx.y;
     if (u >= *a.n_units) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    if (!unit_ok(a, e, row0, nrows)) return;   // tables from an uninitialised workspace must not cause a fault
     const bool shared = e == a.n_experts;
     const int inter = shared ? a.shared_inter : a.inter;
     const int items = inter / 32;
@@ -220,7 +230,7 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
         int g = row0 + c;
         if (shared) return g - nk;
         int i = gather_src[g];
-        return i < 0 ? -1 : i / topk;
+        return (i < 0 || i >= nk) ? -1 : i / topk;
     };
     fill_b_operand(xq, xs, H, nrows, row_src, bq, bsc);
     __syncthreads();
@@ -274,6 +284,7 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
     const int u = blockIdx.y;
     if (u >= *a.n_units) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
     const int inter = shared ? a.shared_inter : a.inter;
     const int H = a.hidden, items = H / 64;
@@ -424,13 +435,15 @@ extern "C" int ferrite_moe_pack_weights(const ferrite_moe_shape* shape, const fe
                                         ferrite_stream_t stream) {
     int rc = check_shape_mfma(shape);
     if (rc) return rc;
-    if (!w || !packed || !w->gate_w || !w->gate_s || !w->up_w || !w->up_s || !w->down_w || !w->down_s)
+    if (!w || !packed || !w->router_w || !w->gate_w || !w->gate_s || !w->up_w || !w->up_s || !w->down_w || !w->down_s)
         return FERRITE_ERR_INVALID_ARG;
     if (shape->shared_inter > 0 && (!w->sh_gate_w || !w->sh_gate_s || !w->sh_up_w || !w->sh_up_s || !w->sh_down_w || !w->sh_down_s))
         return FERRITE_ERR_INVALID_ARG;
     const ferrite_moe_shape& s = *shape;
     PackedLayout L = packed_layout(s);
     hipStream_t st = as_stream(stream);
+    if ((rc = launch_router_transpose(w->router_w, s.n_experts, s.hidden, reinterpret_cast<float*>(packed + L.router_t), st)))
+        return rc;
     PackSrc gu{{w->gate_w, w->up_w}, {w->gate_s, w->up_s}, s.inter, s.hidden, 2, 32};
     if ((rc = pack_one(gu, s.n_experts, packed + L.gu_codes, packed + L.gu_scales, st))) return rc;
     PackSrc dn{{w->down_w, nullptr}, {w->down_s, nullptr}, s.hidden, s.inter, 1, 64};

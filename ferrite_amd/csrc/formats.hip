@@ -2,6 +2,7 @@
 // crates/ferrite-models/src/dsv41/quant.rs (dequant_fp4_row32 :260-278, act_quant_fp8 :190-214) and are
 // bound by HBM traffic: every thread moves 128-bit vectors.
 #include "internal.hpp"
+#include "device_utils.hpp"
 #include "numerics.hpp"
 
 namespace fe {
@@ -36,42 +37,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(const XT* __restrict__ x
                                                         uint8_t* __restrict__ q, uint8_t* __restrict__ scale) {
     int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nblocks) return;
-    float v[32];
-    if constexpr (sizeof(XT) == 4) {
-        const float4* p = reinterpret_cast<const float4*>(x + b * 32);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float4 t = p[i];
-            v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
-        }
-    } else {
-        const uint4* p = reinterpret_cast<const uint4*>(x + b * 32);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint4 t = p[i];
-            uint32_t wds[4] = {t.x, t.y, t.z, t.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                v[8 * i + 2 * j] = u2f(wds[j] << 16);
-                v[8 * i + 2 * j + 1] = u2f(wds[j] & 0xffff0000u);
-            }
-        }
-    }
-    float amax = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
-    uint32_t sb = block_scale_e8m0(amax);
-    float inv = u2f((254u - sb) << 23);   // 2^(127 - sb): exact reciprocal of the power-of-two scale
-    uint32_t out[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        out[i] = e4m3_encode(v[4 * i] * inv) | (e4m3_encode(v[4 * i + 1] * inv) << 8) |
-                 (e4m3_encode(v[4 * i + 2] * inv) << 16) | (e4m3_encode(v[4 * i + 3] * inv) << 24);
-    }
-    uint4* o = reinterpret_cast<uint4*>(q + b * 32);
-    o[0] = make_uint4(out[0], out[1], out[2], out[3]);
-    o[1] = make_uint4(out[4], out[5], out[6], out[7]);
-    scale[b] = (uint8_t)sb;
+    scale[b] = (uint8_t)quant_block32(x + b * 32, q + b * 32);
 }
 
 int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, hipStream_t st) {

@@ -40,6 +40,16 @@ int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* 
                    int32_t* perm_map, int32_t* gather_src, int32_t* active, int32_t* n_active, void* scratch,
                    size_t scratch_bytes, const UnitTables* units, int has_shared, hipStream_t st);
 
+bool head_supported(int n, int H, int E);
+int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
+                    int n, float* logits, float* probs, float* ids_f32, int32_t* ids, uint8_t* xq, uint8_t* xs,
+                    int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
+                    int32_t* active, int32_t* n_active, const UnitTables* units, hipStream_t st);
+int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
+                        hipStream_t st);
+int launch_router_transpose(const float* w, int E, int H, float* dst, hipStream_t st);
+int launch_zero_i32(int32_t* p, int count, hipStream_t st);
+
 // experts_f32.hip (check mode)
 int launch_gate_up_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, const float* x, int n,
                        const int32_t* ids, const int32_t* gather_src, float* act, hipStream_t st);
@@ -54,6 +64,7 @@ struct PackedLayout {
     size_t gu_codes, gu_scales, dn_codes, dn_scales;           // routed experts
     size_t sh_gu_codes, sh_gu_scales, sh_dn_codes, sh_dn_scales; // shared expert
     size_t gu_codes_per_expert, gu_scales_per_expert, dn_codes_per_expert, dn_scales_per_expert;
+    size_t router_t;                                           // k-blocked transpose of the router weight
     size_t total;
 };
 PackedLayout packed_layout(const ferrite_moe_shape& s);

@@ -28,7 +28,7 @@ int check_launch(const char* what) {
 // ---- workspace: fixed offsets for (shape, n, mode) ----
 struct Workspace {
     size_t logits, probs, ids_f32, ids, counts, starts, perm_map, gather_src, active, n_active;
-    size_t unit_expert, unit_row0, unit_rows, n_units, perm_scratch, perm_scratch_bytes;
+    size_t unit_expert, unit_row0, unit_rows, n_units, perm_scratch, perm_scratch_bytes, counters;
     size_t xq, xs, act, act_s, y;
     size_t total;
     int max_units, rows;
@@ -48,6 +48,7 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     w.rows = (int)(nk + (has_shared ? n : 0));
     w.max_units = max_units_for(n, s.topk, s.n_experts, has_shared, 16);
     size_t off = 0;
+    w.counters = bump(off, ((size_t)n + 1) * 4);   // first: ferrite_moe_layer_workspace_init clears it
     w.logits = bump(off, (size_t)n * E * 4);
     w.probs = bump(off, nk * 4);
     w.ids_f32 = bump(off, nk * 4);
@@ -103,6 +104,17 @@ extern "C" size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* sha
     return carve(*shape, n, mode).total;
 }
 
+extern "C" int ferrite_moe_layer_workspace_init(const ferrite_moe_shape* shape, int n, int mode, void* workspace,
+                                                size_t workspace_bytes, ferrite_stream_t stream) {
+    int rc = check_shape(shape, n, mode);
+    if (rc) return rc;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255)) return FERRITE_ERR_INVALID_ARG;
+    Workspace w = carve(*shape, n, mode);
+    if (workspace_bytes < w.total) return FERRITE_ERR_WORKSPACE;
+    return launch_zero_i32(reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + w.counters), n + 1,
+                           as_stream(stream));
+}
+
 extern "C" int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int mode, void* workspace,
                                                 ferrite_moe_workspace_view* v) {
     int rc = check_shape(shape, n, mode);
@@ -124,10 +136,15 @@ extern "C" int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, 
     return FERRITE_OK;
 }
 
-extern "C" int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
-                                       const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
-                                       int out_dtype, int mode, void* workspace, size_t workspace_bytes,
-                                       ferrite_stream_t stream) {
+static int mark(void* const* ev, int i, hipStream_t st) {
+    if (!ev || !ev[i]) return FERRITE_OK;
+    hipError_t e = hipEventRecord(static_cast<hipEvent_t>(ev[i]), st);
+    return e == hipSuccess ? FERRITE_OK : hip_fail(e, "hipEventRecord");
+}
+
+static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts, const uint8_t* packed,
+                          const void* x, int x_dtype, int n, void* out, int out_dtype, int mode, void* workspace,
+                          size_t workspace_bytes, ferrite_stream_t stream, void* const* ev) {
     int rc = check_shape(shape, n, mode);
     if (rc) return rc;
     if (!wts || !wts->router_w || !x || !out || !workspace) return FERRITE_ERR_INVALID_ARG;
@@ -161,37 +178,85 @@ extern "C" int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const fer
     int32_t* gather_src = reinterpret_cast<int32_t*>(b + w.gather_src);
     float* y = reinterpret_cast<float*>(b + w.y);
 
+    UnitTables units{reinterpret_cast<int32_t*>(b + w.unit_expert), reinterpret_cast<int32_t*>(b + w.unit_row0),
+                     reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.n_units), 16,
+                     w.max_units};
+    uint8_t* xq = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xq) : nullptr;
+    uint8_t* xs = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xs) : nullptr;
+    if ((rc = mark(ev, 0, st))) return rc;
+    const bool fused_head = packed != nullptr && head_supported(n, s.hidden, s.n_experts);
+    if (fused_head) {
+        // 1-3 (+ activation quantisation) as one launch
+        PackedLayout L = packed_layout(s);
+        if ((rc = launch_moe_head(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), wts->router_bias, s,
+                                  n, logits, probs, ids_f32, ids, xq, xs, reinterpret_cast<int32_t*>(b + w.counters),
+                                  reinterpret_cast<int32_t*>(b + w.counts), reinterpret_cast<int32_t*>(b + w.starts),
+                                  perm_map, gather_src, reinterpret_cast<int32_t*>(b + w.active),
+                                  reinterpret_cast<int32_t*>(b + w.n_active), &units, st)))
+            return rc;
+        for (int i = 1; i <= 4; ++i)
+            if ((rc = mark(ev, i, st))) return rc;
+    } else {
     // 1. router logits: the reference's sequential-k f32 chain (exec/lib.rs:1107)
-    if ((rc = launch_matmul_exact(x, x_dtype, wts->router_w, nullptr, logits, n, s.hidden, s.n_experts, st))) return rc;
+    if (packed != nullptr && s.hidden % 128 == 0) {
+        PackedLayout L = packed_layout(s);
+        rc = launch_router_chain(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), n, s.hidden,
+                                 s.n_experts, logits, st);
+    } else {
+        rc = launch_matmul_exact(x, x_dtype, wts->router_w, nullptr, logits, n, s.hidden, s.n_experts, st);
+    }
+    if (rc) return rc;
+    if ((rc = mark(ev, 1, st))) return rc;
     // 2. routing (exec/lib.rs:1109-1116); a NULL bias is the reference's zero bias
     if ((rc = ferrite_moe_route(logits, wts->router_bias, n, s.n_experts, s.topk, s.n_group, s.topk_group,
                                 s.routed_scaling, probs, ids_f32, ids, stream)))
         return rc;
+    if ((rc = mark(ev, 2, st))) return rc;
     // 3. permutation by expert + unit tables
-    UnitTables units{reinterpret_cast<int32_t*>(b + w.unit_expert), reinterpret_cast<int32_t*>(b + w.unit_row0),
-                     reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.n_units), 16,
-                     w.max_units};
     if ((rc = launch_permute(ids, n, s.topk, s.n_experts, reinterpret_cast<int32_t*>(b + w.counts),
                              reinterpret_cast<int32_t*>(b + w.starts), perm_map, gather_src,
                              reinterpret_cast<int32_t*>(b + w.active), reinterpret_cast<int32_t*>(b + w.n_active),
                              b + w.perm_scratch, w.perm_scratch_bytes, &units, has_shared, st)))
         return rc;
+    if ((rc = mark(ev, 3, st))) return rc;
+    if (xq) {
+        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq, xs, st))) return rc;
+    }
+    if ((rc = mark(ev, 4, st))) return rc;
+    }
     // 4-5. expert FFNs in grouped order, shared expert as the trailing rows
     if (mode == FERRITE_MODE_F32_CHECK) {
         float* act = reinterpret_cast<float*>(b + w.act);
         if ((rc = launch_gate_up_f32(s, *wts, static_cast<const float*>(x), n, ids, gather_src, act, st))) return rc;
+        if ((rc = mark(ev, 5, st))) return rc;
         if ((rc = launch_down_f32(s, *wts, act, n, ids, gather_src, y, st))) return rc;
     } else {
-        uint8_t* xq = reinterpret_cast<uint8_t*>(b + w.xq);
-        uint8_t* xs = reinterpret_cast<uint8_t*>(b + w.xs);
         uint8_t* act_q = reinterpret_cast<uint8_t*>(b + w.act);
         uint8_t* act_s = reinterpret_cast<uint8_t*>(b + w.act_s);
-        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq, xs, st))) return rc;
         if ((rc = launch_gate_up_mfma(s, packed, xq, xs, n, gather_src, units, act_q, act_s, st))) return rc;
+        if ((rc = mark(ev, 5, st))) return rc;
         if ((rc = launch_down_mfma(s, packed, act_q, act_s, n, units, y, st))) return rc;
     }
+    if ((rc = mark(ev, 6, st))) return rc;
     // 6. weighted combine in slot order + shared expert (exec/lib.rs:1154-1164)
-    return launch_combine(y, probs, perm_map, n, s.topk, s.hidden, has_shared, out, out_dtype, st);
+    if ((rc = launch_combine(y, probs, perm_map, n, s.topk, s.hidden, has_shared, out, out_dtype, st))) return rc;
+    return mark(ev, 7, st);
+}
+
+extern "C" int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
+                                       const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
+                                       int out_dtype, int mode, void* workspace, size_t workspace_bytes,
+                                       ferrite_stream_t stream) {
+    return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, workspace, workspace_bytes, stream,
+                          nullptr);
+}
+
+extern "C" int ferrite_moe_layer_mxfp4_timed(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
+                                             const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
+                                             int out_dtype, int mode, void* workspace, size_t workspace_bytes,
+                                             ferrite_stream_t stream, void* const* stage_events) {
+    return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, workspace, workspace_bytes, stream,
+                          stage_events);
 }
 
 // ---- graph capture (ferrite_graph_begin/end/instantiate/launch, cuda.rs:284-287) ----

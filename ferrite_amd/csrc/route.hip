@@ -1,6 +1,7 @@
 // Router logits (bit-exact sequential-k f32 GEMM), noaux-tc sigmoid group-limited top-k, and the stable
 // token permutation by expert.  gfx950, wave64.
 #include "internal.hpp"
+#include "device_utils.hpp"
 #include "numerics.hpp"
 
 namespace fe {
@@ -152,8 +153,9 @@ __global__ void swiglu_kernel(const float* __restrict__ gate_up, float limit, fl
 }
 
 // ------------------------------------------------------------------------------------------------
-// Routing: one wave per token.  sigmoid -> +bias -> (group top-2 sums -> keep topk_group groups) ->
-// k rounds of wave-wide arg-max on (choice, lower index wins) -> renormalised weights from the raw sigmoid.
+// Routing: one wave per token.  sigmoid -> +bias -> (group top-2 sums -> keep topk_group groups) -> rank of
+// every candidate under (choice desc, index asc) by counting the candidates that beat it -> the topk lowest
+// ranks are the selection, in order -> renormalised weights from the raw sigmoid.
 // Semantics and operation order follow cpu.rs:546-569; ties -> lower index (cpu.rs:560).
 // ------------------------------------------------------------------------------------------------
 constexpr int RT_MAX_E = 512;
@@ -165,52 +167,66 @@ __device__ __forceinline__ uint32_t ordered_u32(float f) {
     return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
 }
 
-__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        unsigned long long o = __shfl_xor(v, off, 64);
-        v = o > v ? o : v;
-    }
-    return v;
+// LDS scratch of one routing wave
+struct RouteScratch {
+    unsigned long long key[RT_MAX_E];
+    float choice[RT_MAX_E];
+    float sel_sig[RT_MAX_K];
+    int sel_id[RT_MAX_K];
+    uint8_t keep[64];
+};
+
+// Loads that must observe stores made by other workgroups of the same kernel.
+__device__ __forceinline__ float load_coherent(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int load_coherent(const int32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
-                                                        const float* __restrict__ bias, int n, int e, int topk,
-                                                        int n_group, int topk_group, float scaling,
-                                                        float* __restrict__ probs, float* __restrict__ ids_f32,
-                                                        int32_t* __restrict__ ids_i32) {
-    __shared__ float choice_lds[4][RT_MAX_E];
-    __shared__ uint8_t keep_lds[4][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int t = blockIdx.x * 4 + wave;
-    const bool live = t < n;
-    const int ni = (e + 63) >> 6;
+// Orders a wave's own LDS traffic: its lanes' earlier writes are visible to its later reads.  The LDS unit
+// executes one wave's instructions in order, so only the compiler has to be kept from reordering.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
 
+// One wave routes one token.  `lg` = the token's e logits.  The scratch is private to the wave, so waves of
+// a block may call this independently of each other.
+template <bool kCoherent>
+__device__ __forceinline__ void route_wave(const float* __restrict__ lg, const float* __restrict__ bias, bool live,
+                                           int e, int topk, int n_group, int topk_group, float scaling,
+                                           RouteScratch& sc, float* __restrict__ probs, float* __restrict__ ids_f32,
+                                           int32_t* __restrict__ ids_i32) {
+    const int lane = threadIdx.x & 63;
+    const int ni = (e + 63) >> 6;
     float sg[RT_NI], ch[RT_NI];
     bool ok[RT_NI];
 #pragma unroll
     for (int i = 0; i < RT_NI; ++i) {
         int j = lane + 64 * i;
         ok[i] = live && i < ni && j < e;
-        float l = ok[i] ? logits[(size_t)t * e + j] : 0.0f;
+        float l = 0.0f;
+        if (ok[i]) l = kCoherent ? load_coherent(lg + j) : lg[j];
         sg[i] = sigmoid_ref(l);
         ch[i] = ok[i] ? fadd(sg[i], bias ? bias[j] : 0.0f) : 0.0f;
     }
+    if (lane < RT_MAX_K) { sc.sel_id[lane] = -1; sc.sel_sig[lane] = 0.0f; }
 
     if (n_group > 1) {
         const int gs = e / n_group;
 #pragma unroll
         for (int i = 0; i < RT_NI; ++i) {
             int j = lane + 64 * i;
-            if (i < ni && j < e) choice_lds[wave][j] = ch[i];
+            if (i < ni && j < e) sc.choice[j] = ch[i];
         }
-        __syncthreads();
+        wave_sync();
         // lane g scores group g: largest + second largest choice (largest first)
         float gscore = 0.0f;
         if (lane < n_group) {
             float m1 = u2f(0xff800000u), m2 = u2f(0xff800000u);
             for (int j = lane * gs; j < (lane + 1) * gs; ++j) {
-                float c = choice_lds[wave][j];
+                float c = sc.choice[j];
                 if (c > m1) { m2 = m1; m1 = c; }
                 else if (c > m2) m2 = c;
             }
@@ -222,67 +238,78 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
             float s2 = __shfl(gscore, g2, 64);
             rank += (s2 > gscore || (s2 == gscore && g2 < lane)) ? 1 : 0;
         }
-        if (lane < n_group) keep_lds[wave][lane] = rank < topk_group ? 1 : 0;
-        __syncthreads();
+        if (lane < n_group) sc.keep[lane] = rank < topk_group ? 1 : 0;
+        wave_sync();
 #pragma unroll
         for (int i = 0; i < RT_NI; ++i) {
             int j = lane + 64 * i;
-            if (ok[i] && !keep_lds[wave][j / gs]) ok[i] = false;
+            if (ok[i] && !sc.keep[j / gs]) ok[i] = false;
         }
     }
 
+    // key = (order-preserving bits of choice, inverted index): larger key = earlier in the reference's sort
     unsigned long long key[RT_NI];
 #pragma unroll
     for (int i = 0; i < RT_NI; ++i) {
         uint32_t j = lane + 64 * i;
         key[i] = ok[i] ? (((unsigned long long)ordered_u32(ch[i]) << 32) | (0xFFFFFFFFu - j)) : 0ull;
+        if (i < ni && (int)j < e) sc.key[j] = key[i];
     }
-
-    int my_id = -1;
-    float my_sig = 0.0f;
-    for (int r = 0; r < topk; ++r) {
-        unsigned long long best = 0ull;
+    wave_sync();
+    int rank[RT_NI];
 #pragma unroll
-        for (int i = 0; i < RT_NI; ++i) best = key[i] > best ? key[i] : best;
-        best = wave_max_u64(best);
-        uint32_t j = 0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFull);
-        int wi = (int)(j >> 6), wl = (int)(j & 63);
-        float sv = 0.0f;
+    for (int i = 0; i < RT_NI; ++i) rank[i] = 0;
+    for (int j2 = 0; j2 < e; ++j2) {
+        const unsigned long long kj = sc.key[j2];   // same address in every lane: an LDS broadcast
 #pragma unroll
-        for (int i = 0; i < RT_NI; ++i) {
-            if (i == wi) {
-                sv = sg[i];
-                if (lane == wl) key[i] = 0ull;
-            }
-        }
-        sv = __shfl(sv, wl, 64);
-        if (lane == r) {
-            my_id = best ? (int)j : -1;
-            my_sig = sv;
+        for (int i = 0; i < RT_NI; ++i) rank[i] += kj > key[i] ? 1 : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < RT_NI; ++i) {
+        if (key[i] != 0ull && rank[i] < topk) {
+            sc.sel_id[rank[i]] = lane + 64 * i;
+            sc.sel_sig[rank[i]] = sg[i];
         }
     }
+    wave_sync();
     // cpu.rs:562-568: sum in selection order, then sig / (sum + f32::EPSILON) * scale
     float sum = 0.0f;
-    for (int r = 0; r < topk; ++r) sum = fadd(sum, __shfl(my_sig, r, 64));
+    for (int r = 0; r < topk; ++r) sum = fadd(sum, sc.sel_sig[r]);
     if (live && lane < topk) {
-        size_t o = (size_t)t * topk + lane;
-        probs[o] = fmul(fdiv(my_sig, fadd(sum, 1.1920928955078125e-07f)), scaling);
-        if (ids_f32) ids_f32[o] = (float)my_id;
-        if (ids_i32) ids_i32[o] = my_id;
+        const float my_sig = sc.sel_sig[lane];
+        const int my_id = sc.sel_id[lane];
+        probs[lane] = fmul(fdiv(my_sig, fadd(sum, 1.1920928955078125e-07f)), scaling);
+        if (ids_f32) ids_f32[lane] = (float)my_id;
+        if (ids_i32) ids_i32[lane] = my_id;
     }
+}
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
+                                                        const float* __restrict__ bias, int n, int e, int topk,
+                                                        int n_group, int topk_group, float scaling,
+                                                        float* __restrict__ probs, float* __restrict__ ids_f32,
+                                                        int32_t* __restrict__ ids_i32) {
+    __shared__ RouteScratch scratch[4];
+    const int wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    const bool live = t < n;
+    const size_t tt = live ? t : 0;
+    route_wave<false>(logits + tt * e, bias, live, e, topk, n_group, topk_group, scaling, scratch[wave],
+                      probs + tt * topk, ids_f32 ? ids_f32 + tt * topk : nullptr,
+                      ids_i32 ? ids_i32 + tt * topk : nullptr);
 }
 
 // ------------------------------------------------------------------------------------------------
 // Stable permutation by expert.  Every token holds each expert at most once, so the assignments of expert e
 // in ascending flat index are its tokens in ascending order: rank = number of earlier tokens that chose e.
-// Tokens are cut into chunks of 64 (one wave); per (expert, chunk) a 64-bit membership mask is built with
-// LDS atomics; a per-expert prefix over chunks plus a popcount below the token's bit gives the rank, and an
-// exclusive scan of the per-expert totals gives the expert's first grouped row.  No global atomics and no
-// dependence on scheduling: the tables are a pure function of ids.
+// Tokens are cut into chunks of 64; per (expert, chunk) a 64-bit membership mask is built with LDS atomics;
+// a per-expert prefix over chunks plus a popcount below the token's bit gives the rank, and an exclusive
+// scan of the per-expert totals gives the expert's first grouped row.  No global atomics and no dependence
+// on scheduling: the tables are a pure function of ids.
 //   phase A: masks    phase B: per-expert chunk prefixes, expert scan, active list, unit tables
 //   phase C: scatter
-// n <= 1024 runs A,B,C in one block with the masks in LDS; larger n uses three launches with the masks in
-// the caller's scratch.
+// Small n runs A,B,C in one block with the masks in LDS; larger n uses three launches with the masks in the
+// caller's scratch.
 // ------------------------------------------------------------------------------------------------
 constexpr int PM_MAX_E = 512;
 constexpr int PM_SMALL_N = 1024;
@@ -364,24 +391,33 @@ __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t*
     }
 }
 
-__global__ __launch_bounds__(1024) void permute_small_kernel(PermArgs a) {
-    extern __shared__ unsigned long long pm_lds[];
+static inline size_t perm_block_lds_bytes(int n, int n_experts) {
+    size_t nchunk = ((size_t)n + 63) / 64;
+    return (size_t)n_experts * nchunk * 12 + (size_t)(2 * n_experts + 1) * 4;
+}
+
+// The whole permutation by one workgroup (any multiple of 64 threads) or, with kWaveScope, by a single wave
+// of a larger workgroup.  lds: perm_block_lds_bytes.
+template <bool kCoherent, bool kWaveScope>
+__device__ void permute_in_block(const PermArgs& a, unsigned long long* lds) {
     const int E = a.n_experts, n = a.n, k = a.topk;
     const int nchunk = (n + 63) >> 6;
-    unsigned long long* mask = pm_lds;                                   // [E][nchunk]
+    unsigned long long* mask = lds;                                      // [E][nchunk]
     int32_t* offs = reinterpret_cast<int32_t*>(mask + (size_t)E * nchunk);  // [E][nchunk]
     int32_t* cnt = offs + (size_t)E * nchunk;                            // [E]
     int32_t* starts_lds = cnt + E;                                       // [E+1]
-    const int tid = threadIdx.x;
-    for (int i = tid; i < E * nchunk; i += blockDim.x) mask[i] = 0ull;
-    __syncthreads();
-    for (int t = tid; t < n; t += blockDim.x)
-        for (int j = 0; j < k; ++j) {
-            int e = a.ids[(size_t)t * k + j];
-            if (e >= 0 && e < E) atomicOr(&mask[(size_t)e * nchunk + (t >> 6)], 1ull << (t & 63));
-        }
-    __syncthreads();
-    for (int e = tid; e < E; e += blockDim.x) {
+    const int tid = kWaveScope ? (threadIdx.x & 63) : threadIdx.x, nthr = kWaveScope ? 64 : blockDim.x;
+    auto sync = [] { if constexpr (kWaveScope) wave_sync(); else __syncthreads(); };
+    auto id_at = [&](int i) -> int { return kCoherent ? load_coherent(a.ids + i) : a.ids[i]; };
+    for (int i = tid; i < E * nchunk; i += nthr) mask[i] = 0ull;
+    sync();
+    for (int i = tid; i < n * k; i += nthr) {
+        int t = i / k;
+        int e = id_at(i);
+        if (e >= 0 && e < E) atomicOr(&mask[(size_t)e * nchunk + (t >> 6)], 1ull << (t & 63));
+    }
+    sync();
+    for (int e = tid; e < E; e += nthr) {
         int run = 0;
         for (int c = 0; c < nchunk; ++c) {
             offs[(size_t)e * nchunk + c] = run;
@@ -389,21 +425,25 @@ __global__ __launch_bounds__(1024) void permute_small_kernel(PermArgs a) {
         }
         cnt[e] = run;
     }
-    __syncthreads();
+    sync();
     if (tid < 64) perm_expert_scan(a, cnt, starts_lds);
-    __syncthreads();
+    sync();
     const int total = starts_lds[E];
-    for (int t = tid; t < n; t += blockDim.x)
-        for (int j = 0; j < k; ++j) {
-            int i = t * k + j;
-            int e = a.ids[i];
-            if (e < 0 || e >= E) { a.perm_map[i] = -1; continue; }
-            unsigned long long m = mask[(size_t)e * nchunk + (t >> 6)];
-            int g = starts_lds[e] + offs[(size_t)e * nchunk + (t >> 6)] + __popcll(m & ((1ull << (t & 63)) - 1ull));
-            a.perm_map[i] = g;
-            a.gather_src[g] = i;
-        }
-    for (int g = total + tid; g < n * k; g += blockDim.x) a.gather_src[g] = -1;
+    for (int i = tid; i < n * k; i += nthr) {
+        int t = i / k;
+        int e = id_at(i);
+        if (e < 0 || e >= E) { a.perm_map[i] = -1; continue; }
+        unsigned long long m = mask[(size_t)e * nchunk + (t >> 6)];
+        int g = starts_lds[e] + offs[(size_t)e * nchunk + (t >> 6)] + __popcll(m & ((1ull << (t & 63)) - 1ull));
+        a.perm_map[i] = g;
+        a.gather_src[g] = i;
+    }
+    for (int g = total + tid; g < n * k; g += nthr) a.gather_src[g] = -1;
+}
+
+__global__ __launch_bounds__(1024) void permute_small_kernel(PermArgs a) {
+    extern __shared__ unsigned long long pm_lds[];
+    permute_in_block<false, false>(a, pm_lds);
 }
 
 // large-n phase A: one wave per 64-token chunk
@@ -464,6 +504,285 @@ __global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const 
     a.gather_src[g] = (int)i;
 }
 
+// ------------------------------------------------------------------------------------------------
+// The head of the layer as ONE launch (decode-sized batches), or the router GEMM alone (kFused = false).
+//   blocks (eb, tb), eb < eblocks : router logits of tokens [4 tb, 4 tb + 4) (one per wave) for experts
+//                                   [64 eb, 64 eb + 64) (one per lane): the reference's sequential chain.  The
+//                                   router weight comes from its k-blocked transpose [H/4][Epad][4], so a
+//                                   128-k chunk of the block's 64 experts is one contiguous 32 KiB; chunks of
+//                                   it and of the four x rows are staged in LDS (two buffers) behind a
+//                                   two-chunk register prefetch, so the chains never wait on memory
+//   blocks (eblocks, tb)          : e4m3-per-32 quantisation of those four x rows (off the critical path)
+//   last logits wave of a token   : routes the token (arrival counter per token)
+//   last routed token             : builds the permutation and unit tables, then clears the counters so the
+//                                   next launch (or graph replay) starts clean
+// counters[0] = routed tokens, counters[1 + t] = logits blocks of token t that have arrived; all zero on entry.
+// ------------------------------------------------------------------------------------------------
+constexpr int HEAD_MAX_N = 256;
+constexpr int HD_TT = 4;          // tokens per block
+constexpr int HD_C4 = 32;         // float4 (4 k) per chunk and expert
+constexpr size_t HD_W_BYTES = (size_t)HD_C4 * 64 * 16;        // 32 KiB
+constexpr size_t HD_X_BYTES = (size_t)HD_TT * HD_C4 * 16;     // 2 KiB
+constexpr size_t HD_STAGE_BYTES = 2 * (HD_W_BYTES + HD_X_BYTES);
+
+struct HeadArgs {
+    const void* x;
+    const float* wt;      // [H/4][Epad][4]
+    const float* bias;
+    int n, H, E, Epad, topk, n_group, topk_group;
+    float scaling;
+    float *logits, *probs, *ids_f32;
+    int32_t* ids;
+    uint8_t *xq, *xs;     // may be NULL: no quantisation blocks are launched then
+    int32_t* counters;    // [1 + n]
+    PermArgs perm;
+};
+
+struct HeadStage {
+    float4 w[8];
+    float4 x;
+};
+
+template <typename XT>
+__device__ __forceinline__ void head_fetch(HeadStage& st, int c, int tid, const float4* __restrict__ wsrc, int Epad,
+                                           const XT* __restrict__ xrow) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+        const int i = tid + 256 * p;
+        st.w[p] = wsrc[(size_t)(c * HD_C4 + (i >> 6)) * Epad + (i & 63)];
+    }
+    const int k4 = c * HD_C4 + (tid & 31);   // threads >= 128 load a duplicate that is never stored
+    if constexpr (sizeof(XT) == 4) {
+        st.x = reinterpret_cast<const float4*>(xrow)[k4];
+    } else {
+        uint2 q = reinterpret_cast<const uint2*>(xrow)[k4];
+        st.x = make_float4(u2f(q.x << 16), u2f(q.x & 0xffff0000u), u2f(q.y << 16), u2f(q.y & 0xffff0000u));
+    }
+}
+
+__device__ __forceinline__ void head_stash(const HeadStage& st, int buf, int tid, float4* w_lds, float4* x_lds) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) w_lds[(size_t)buf * HD_C4 * 64 + tid + 256 * p] = st.w[p];
+    if (tid < HD_TT * HD_C4) x_lds[buf * HD_TT * HD_C4 + tid] = st.x;
+}
+
+// The chain over one staged chunk: 8 groups of 4 float4 in a rolled loop over pairs of groups with two named
+// register buffers, so that the LDS reads of a group are in flight while the previous group's 16 chain steps
+// execute (fully unrolled, the compiler hoists every read of the chunk and runs out of registers).
+__device__ __forceinline__ float head_chain(float s, const float4* wl, const float4* xl) {
+    constexpr int G = 4;
+    constexpr int NG = HD_C4 / G;
+    float4 wA[G], xA[G], wB[G], xB[G];
+#pragma unroll
+    for (int j = 0; j < G; ++j) { wA[j] = wl[j * 64]; xA[j] = xl[j]; }
+#pragma nounroll
+    for (int g = 0; g < NG; g += 2) {
+#pragma unroll
+        for (int j = 0; j < G; ++j) { wB[j] = wl[((g + 1) * G + j) * 64]; xB[j] = xl[(g + 1) * G + j]; }
+#pragma unroll
+        for (int j = 0; j < G; ++j) {
+            s = fadd(s, fmul(xA[j].x, wA[j].x));
+            s = fadd(s, fmul(xA[j].y, wA[j].y));
+            s = fadd(s, fmul(xA[j].z, wA[j].z));
+            s = fadd(s, fmul(xA[j].w, wA[j].w));
+        }
+        const int gn = g + 2 < NG ? g + 2 : NG - 1;   // the last pass re-reads a group it does not use
+#pragma unroll
+        for (int j = 0; j < G; ++j) { wA[j] = wl[(gn * G + j) * 64]; xA[j] = xl[gn * G + j]; }
+#pragma unroll
+        for (int j = 0; j < G; ++j) {
+            s = fadd(s, fmul(xB[j].x, wB[j].x));
+            s = fadd(s, fmul(xB[j].y, wB[j].y));
+            s = fadd(s, fmul(xB[j].z, wB[j].z));
+            s = fadd(s, fmul(xB[j].w, wB[j].w));
+        }
+    }
+    return s;
+}
+
+template <typename XT, bool kFused>
+__global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
+    extern __shared__ __align__(16) unsigned char head_lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int eb = blockIdx.x, t0 = blockIdx.y * HD_TT;
+    const int eblocks = a.Epad >> 6;
+    const int H = a.H;
+    const XT* xbase = static_cast<const XT*>(a.x);
+    if (eb == eblocks) {
+        const int bpr = H / 32;   // blocks per row
+        for (int i = tid; i < HD_TT * bpr; i += 256) {
+            const int t = t0 + i / bpr, b = i % bpr;
+            if (t < a.n)
+                a.xs[(size_t)t * bpr + b] = (uint8_t)quant_block32(xbase + (size_t)t * H + b * 32,
+                                                                   a.xq + (size_t)t * H + b * 32);
+        }
+        return;
+    }
+    float4* w_lds = reinterpret_cast<float4*>(head_lds);                      // [2][HD_C4][64]
+    float4* x_lds = reinterpret_cast<float4*>(head_lds + 2 * HD_W_BYTES);     // [2][HD_TT][HD_C4]
+    const int nk4 = H / 4;
+    const int nchunk = nk4 / HD_C4;
+    const float4* wsrc = reinterpret_cast<const float4*>(a.wt) + (size_t)eb * 64;
+
+    // H is a multiple of 128 here, so every chunk is full; rows past n are clamped to row n-1 (their results
+    // are never stored), which keeps the staging free of branches
+    const int xt = min(t0 + ((tid >> 5) & (HD_TT - 1)), a.n - 1);
+    const XT* xrow = xbase + (size_t)xt * H;
+    const float4* wl0 = w_lds + lane;
+    const float4* xl0 = x_lds + wave * HD_C4;
+    HeadStage sa, sb;
+    float s = 0.0f;
+    // The scheduling barriers pin the order "issue the loads of chunk c+2 -> chain over chunk c -> store chunk
+    // c+1 to LDS": without them the stores (and the wait for their global loads) drift in front of the chain.
+    head_fetch(sa, 0, tid, wsrc, a.Epad, xrow);
+    head_fetch(sb, nchunk > 1 ? 1 : 0, tid, wsrc, a.Epad, xrow);
+    head_stash(sa, 0, tid, w_lds, x_lds);
+    __syncthreads();
+    for (int c = 0; c < nchunk; c += 2) {
+        head_fetch(sa, min(c + 2, nchunk - 1), tid, wsrc, a.Epad, xrow);
+        __builtin_amdgcn_sched_barrier(0);
+        s = head_chain(s, wl0, xl0);
+        __builtin_amdgcn_sched_barrier(0);
+        head_stash(sb, 1, tid, w_lds, x_lds);
+        __syncthreads();
+        if (c + 1 < nchunk) {
+            head_fetch(sb, min(c + 3, nchunk - 1), tid, wsrc, a.Epad, xrow);
+            __builtin_amdgcn_sched_barrier(0);
+            s = head_chain(s, wl0 + (size_t)HD_C4 * 64, xl0 + HD_TT * HD_C4);
+            __builtin_amdgcn_sched_barrier(0);
+            head_stash(sa, 0, tid, w_lds, x_lds);
+            __syncthreads();
+        }
+    }
+    const int t = t0 + wave, e = eb * 64 + lane;
+    const bool live = t < a.n;
+    if (live && e < a.E) a.logits[(size_t)t * a.E + e] = s;
+    if constexpr (!kFused) return;
+    if (!live) return;   // wave-uniform; no block-wide barrier follows
+
+    // arrival: the stores above are made visible before the counter moves
+    __threadfence();
+    int last = 0;
+    if (lane == 0) last = atomicAdd(&a.counters[1 + t], 1) == eblocks - 1;
+    last = __shfl(last, 0, 64);
+    if (!last) return;
+    __threadfence();
+    // the staging buffers are dead for this wave; each wave takes a private slice of them as scratch
+    RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds + (size_t)wave * sizeof(RouteScratch));
+    route_wave<true>(a.logits + (size_t)t * a.E, a.bias, true, a.E, a.topk, a.n_group, a.topk_group, a.scaling, sc,
+                     a.probs + (size_t)t * a.topk, a.ids_f32 + (size_t)t * a.topk, a.ids + (size_t)t * a.topk);
+    __threadfence();
+    last = 0;
+    if (lane == 0) last = atomicAdd(&a.counters[0], 1) == a.n - 1;
+    last = __shfl(last, 0, 64);
+    if (!last) return;
+    __threadfence();
+    // the permutation scratch sits above the four routing scratches (another wave may still be routing)
+    permute_in_block<true, true>(a.perm, reinterpret_cast<unsigned long long*>(head_lds + 4 * sizeof(RouteScratch)));
+    for (int i = lane; i < a.n + 1; i += 64) a.counters[i] = 0;
+}
+
+static size_t head_lds_bytes(int n, int E, bool fused) {
+    size_t b = HD_STAGE_BYTES;
+    if (fused) {
+        size_t p = 4 * sizeof(RouteScratch) + perm_block_lds_bytes(n, E);
+        if (p > b) b = p;
+    }
+    return b;
+}
+
+bool head_supported(int n, int H, int E) {
+    return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, E, true) <= 150 * 1024;
+}
+
+template <typename K>
+static int raise_lds(K kernel, size_t bytes, size_t* raised) {
+    if (bytes <= 64 * 1024 || bytes <= *raised) return FERRITE_OK;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+    *raised = bytes;
+    return FERRITE_OK;
+}
+
+template <typename XT, bool kFused>
+static int launch_head_t(const HeadArgs& a, dim3 grid, size_t lds, hipStream_t st) {
+    static size_t raised = 0;
+    int rc = raise_lds(moe_head_kernel<XT, kFused>, lds, &raised);
+    if (rc) return rc;
+    moe_head_kernel<XT, kFused><<<grid, 256, lds, st>>>(a);
+    return check_launch("moe_head");
+}
+
+int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
+                    int n, float* logits, float* probs, float* ids_f32, int32_t* ids, uint8_t* xq, uint8_t* xs,
+                    int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
+                    int32_t* active, int32_t* n_active, const UnitTables* units, hipStream_t st) {
+    if (!head_supported(n, s.hidden, s.n_experts)) return FERRITE_DECLINED;
+    HeadArgs a{};
+    a.x = x; a.wt = router_t; a.bias = bias;
+    a.n = n; a.H = s.hidden; a.E = s.n_experts; a.Epad = (s.n_experts + 63) / 64 * 64; a.topk = s.topk;
+    a.n_group = (s.n_group > 1 && s.topk_group < s.n_group) ? s.n_group : 1;
+    a.topk_group = s.topk_group; a.scaling = s.routed_scaling;
+    a.logits = logits; a.probs = probs; a.ids_f32 = ids_f32; a.ids = ids; a.xq = xq; a.xs = xs; a.counters = counters;
+    PermArgs& p = a.perm;
+    p.ids = ids; p.n = n; p.topk = s.topk; p.n_experts = s.n_experts;
+    p.counts = counts; p.starts = starts; p.perm_map = perm_map; p.gather_src = gather_src;
+    p.active = active; p.n_active = n_active; p.has_shared = s.shared_inter > 0;
+    if (units) {
+        p.unit_expert = units->unit_expert; p.unit_row0 = units->unit_row0; p.unit_rows = units->unit_rows;
+        p.n_units = units->n_units; p.unit_cap = units->unit_rows_cap; p.max_units = units->max_units;
+    }
+    dim3 grid(a.Epad / 64 + (xq ? 1 : 0), (n + HD_TT - 1) / HD_TT);
+    const size_t lds = head_lds_bytes(n, s.n_experts, true);
+    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, grid, lds, st);
+    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, true>(a, grid, lds, st);
+    return FERRITE_ERR_INVALID_ARG;
+}
+
+// Router GEMM alone from the transposed weight (any n): logits only.
+int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
+                        hipStream_t st) {
+    if (H % 128 != 0 || n <= 0) return FERRITE_DECLINED;
+    HeadArgs a{};
+    a.x = x; a.wt = router_t; a.n = n; a.H = H; a.E = E; a.Epad = (E + 63) / 64 * 64; a.logits = logits;
+    dim3 grid(a.Epad / 64, (n + HD_TT - 1) / HD_TT);
+    const size_t lds = head_lds_bytes(n, E, false);
+    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, false>(a, grid, lds, st);
+    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, false>(a, grid, lds, st);
+    return FERRITE_ERR_INVALID_ARG;
+}
+
+// router weight [E][H] -> k-blocked transpose [H/4][Epad][4], zero padded
+__global__ __launch_bounds__(256) void router_transpose_kernel(const float* __restrict__ w, int E, int Epad, int H,
+                                                               float4* __restrict__ dst) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (size_t)(H / 4) * Epad) return;
+    int e = (int)(idx % Epad);
+    size_t k4 = idx / Epad;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (e < E) v = *reinterpret_cast<const float4*>(w + (size_t)e * H + k4 * 4);
+    dst[idx] = v;
+}
+
+int launch_router_transpose(const float* w, int E, int H, float* dst, hipStream_t st) {
+    const int Epad = (E + 63) / 64 * 64;
+    size_t total = (size_t)(H / 4) * Epad;
+    router_transpose_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(w, E, Epad, H, reinterpret_cast<float4*>(dst));
+    return check_launch("router_transpose");
+}
+
+__global__ void zero_i32_kernel(int32_t* p, int count) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) p[i] = 0;
+}
+
+int launch_zero_i32(int32_t* p, int count, hipStream_t st) {
+    if (count <= 0) return FERRITE_OK;
+    zero_i32_kernel<<<(count + 255) / 256, 256, 0, st>>>(p, count);
+    return check_launch("zero_i32");
+}
+
 static size_t perm_scratch_bytes(int n, int n_experts) {
     size_t nchunk = ((size_t)n + 63) / 64;
     return (size_t)n_experts * nchunk * (8 + 4) + 64;
@@ -482,7 +801,7 @@ int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* 
         a.n_units = units->n_units; a.unit_cap = units->unit_rows_cap; a.max_units = units->max_units;
     }
     const int nchunk = (n + 63) / 64;
-    const size_t lds = (size_t)n_experts * nchunk * 12 + (size_t)(2 * n_experts + 1) * 4;
+    const size_t lds = perm_block_lds_bytes(n, n_experts);
     if (n <= PM_SMALL_N && lds <= 60 * 1024) {
         permute_small_kernel<<<1, 1024, lds, st>>>(a);
         return check_launch("permute_small");

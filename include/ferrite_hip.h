@@ -142,6 +142,11 @@ typedef struct ferrite_moe_workspace_view {
 } ferrite_moe_workspace_view;
 
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
+/* Must run once on a freshly allocated workspace before its first layer call (it clears the arrival counters
+ * the fused routing kernel keeps there; the kernel leaves them cleared, so replays need no further call).
+ * Workspaces are owned by the caller like every other buffer (DevBuf pool, cuda.rs:558-744). */
+int ferrite_moe_layer_workspace_init(const ferrite_moe_shape* shape, int n, int mode, void* workspace,
+                                     size_t workspace_bytes, ferrite_stream_t stream);
 int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int mode, void* workspace,
                                      ferrite_moe_workspace_view* view_host);
 
@@ -152,6 +157,17 @@ int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int 
 int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, const uint8_t* packed,
                             const void* x, int x_dtype, int n, void* out, int out_dtype, int mode,
                             void* workspace, size_t workspace_bytes, ferrite_stream_t stream);
+
+/* The same layer with HIP events recorded on `stream` at the stage boundaries, the counterpart of the
+ * reference's FERRITE_TIMING probes (crates/ferrite-exec/src/lib.rs:1184-1299).  stage_events_host is a host
+ * array of FERRITE_MOE_STAGE_EVENTS hipEvent_t handles (any may be NULL): [0] before the router GEMM, then
+ * after: [1] router GEMM, [2] routing, [3] permutation, [4] activation quantisation (== [3] in f32 mode),
+ * [5] gate/up GEMM + SwiGLU, [6] down GEMM, [7] combine.  Not capturable. */
+#define FERRITE_MOE_STAGE_EVENTS 8
+int ferrite_moe_layer_mxfp4_timed(const ferrite_moe_shape* shape, const ferrite_moe_weights* w,
+                                  const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
+                                  int out_dtype, int mode, void* workspace, size_t workspace_bytes,
+                                  ferrite_stream_t stream, void* const* stage_events_host);
 
 /* ---- graph capture: ferrite_graph_begin/end/instantiate/launch (cuda.rs:284-287) ---- */
 int ferrite_graph_begin(ferrite_stream_t stream);

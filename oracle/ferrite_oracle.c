@@ -151,19 +151,28 @@ void fo_act_quant_fp4(const float* x, size_t len, int block, int round_scale, ui
     free(nib);
 }
 
-/* quant.rs:260-278: low nibble = even column (quant.rs:57-68) */
-void fo_dequant_fp4_row32(const uint8_t* w, const uint8_t* scale, size_t out, size_t inn, float* dst) {
-    const size_t B = 32;
-    size_t nb_in = inn / B;
+/* quant.rs:260-278: low nibble = even column (quant.rs:57-68).  Same per-element arithmetic as the reference
+ * (table[code] * 2^(scale-127)), walked one 32-column block at a time; rows are independent, so `nt` > 1
+ * splits them over threads. */
+static void dequant_fp4_row32_mt(const uint8_t* w, const uint8_t* scale, size_t out, size_t inn, float* dst, int nt) {
+    const size_t nb_in = inn / 32;
+#pragma omp parallel for num_threads(nt > 1 ? nt : 1) schedule(static)
     for (size_t r = 0; r < out; ++r) {
         const uint8_t* row = w + r * (inn / 2);
-        for (size_t c = 0; c < inn; ++c) {
-            uint8_t byte = row[c / 2];
-            uint8_t code = (c % 2 == 0) ? (byte & 0x0F) : ((byte >> 4) & 0x0F);
-            float s = fo_ue8m0_decode(scale[r * nb_in + c / B]);
-            dst[r * inn + c] = fo_e2m1_decode(code) * s;
+        float* d = dst + r * inn;
+        for (size_t b = 0; b < nb_in; ++b) {
+            float s = fo_ue8m0_decode(scale[r * nb_in + b]);
+            for (size_t i = 0; i < 16; ++i) {
+                uint8_t byte = row[b * 16 + i];
+                d[b * 32 + 2 * i] = FO_FP4_TABLE[byte & 0x0F] * s;
+                d[b * 32 + 2 * i + 1] = FO_FP4_TABLE[(byte >> 4) & 0x0F] * s;
+            }
         }
     }
+}
+
+void fo_dequant_fp4_row32(const uint8_t* w, const uint8_t* scale, size_t out, size_t inn, float* dst) {
+    dequant_fp4_row32_mt(w, scale, out, inn, dst, 1);
 }
 
 /* ------------------------------------------------------------- CpuBackend ops */
@@ -494,9 +503,9 @@ int fo_moe_ffn_mxfp4(const fo_moe_cfg* cfg, const fo_moe_weights* w, const float
             for (int j = 0; j < K; ++j)
                 if ((int)ids[(size_t)sel[r] * K + j] == e) { rows[m] = sel[r]; ydst[m] = y + ((size_t)r * K + j) * H; ++m; }
         if (m == 0) continue;
-        fo_dequant_fp4_row32(w->gate_w + e * gsz, w->gate_s + e * gss, (size_t)I, (size_t)H, wg);
-        fo_dequant_fp4_row32(w->up_w + e * gsz, w->up_s + e * gss, (size_t)I, (size_t)H, wu);
-        fo_dequant_fp4_row32(w->down_w + e * dsz, w->down_s + e * dss, (size_t)H, (size_t)I, wd);
+        dequant_fp4_row32_mt(w->gate_w + e * gsz, w->gate_s + e * gss, (size_t)I, (size_t)H, wg, nt);
+        dequant_fp4_row32_mt(w->up_w + e * gsz, w->up_s + e * gss, (size_t)I, (size_t)H, wu, nt);
+        dequant_fp4_row32_mt(w->down_w + e * dsz, w->down_s + e * dss, (size_t)H, (size_t)I, wd, nt);
         expert_rows(cfg, xin, rows, m, wg, wu, wd, I, ydst);
     }
 
@@ -504,9 +513,9 @@ int fo_moe_ffn_mxfp4(const fo_moe_cfg* cfg, const fo_moe_weights* w, const float
     float* shared = NULL;
     if (Is > 0) {
         shared = (float*)malloc(sizeof(float) * (size_t)ns * H);
-        fo_dequant_fp4_row32(w->sh_gate_w, w->sh_gate_s, (size_t)Is, (size_t)H, wg);
-        fo_dequant_fp4_row32(w->sh_up_w, w->sh_up_s, (size_t)Is, (size_t)H, wu);
-        fo_dequant_fp4_row32(w->sh_down_w, w->sh_down_s, (size_t)H, (size_t)Is, wd);
+        dequant_fp4_row32_mt(w->sh_gate_w, w->sh_gate_s, (size_t)Is, (size_t)H, wg, nt);
+        dequant_fp4_row32_mt(w->sh_up_w, w->sh_up_s, (size_t)Is, (size_t)H, wu, nt);
+        dequant_fp4_row32_mt(w->sh_down_w, w->sh_down_s, (size_t)H, (size_t)Is, wd, nt);
         for (int r = 0; r < ns; ++r) { rows[r] = sel[r]; ydst[r] = shared + (size_t)r * H; }
         expert_rows(cfg, xin, rows, ns, wg, wu, wd, Is, ydst);
     }

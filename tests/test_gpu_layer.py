@@ -133,3 +133,32 @@ def test_layer_graph_capture_replays(hip, oracle):
         assert hip.end_verify()
         assert torch.equal(out_static, eager)
     hip.graph_destroy(trace)
+
+
+def test_layer_unfused_head_path(hip, oracle):
+    """More tokens than the fused routing kernel takes (n > 256): separate router GEMM, routing, three-phase
+    permutation and quantisation launches; results must not depend on which head ran."""
+    cfg = synth.MoeConfig(300, 256, 16, 4, 128, 128, 4, 2)
+    inp = synth.make_inputs(cfg, seed=9)
+    layer = hip.load_moe_layer(inp)
+    ref32 = oracle.moe_ffn_mxfp4(inp, n_threads=8)
+    out, v = run_layer(hip, layer, inp.x, MODE_F32_CHECK)
+    check_routing(v, ref32, oracle, cfg)
+    assert max_abs_rel(out, ref32["out"]) <= TOL_F32
+    out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    check_routing(v, ref32, oracle, cfg)
+    assert max_abs_rel(out, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
+
+
+def test_layer_repeated_calls_same_workspace(hip, oracle):
+    """The fused routing kernel keeps arrival counters in the workspace and must leave them cleared."""
+    inp = synth.make_inputs(synth.CONFIGS["c0"].with_tokens(40), seed=3)
+    layer = hip.load_moe_layer(inp)
+    ref = oracle.moe_ffn_mxfp4(inp, act_mode=1)
+    first = None
+    for _ in range(5):
+        out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+        check_routing(v, ref, oracle, inp.cfg)
+        first = out if first is None else first
+        assert np.array_equal(out, first)
+    assert max_abs_rel(first, ref["out"]) <= TOL_MFMA
