@@ -87,6 +87,8 @@ def main():
     ap.add_argument("--tokens", type=int, default=0, help="override the token count of the config")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of graph replays")
+    ap.add_argument("--calib-copy-mib", type=int, default=0,
+                    help="also run a plain device copy of this many MiB (a counter calibration point for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -114,6 +116,14 @@ def main():
 
     def step():
         hip.moe_layer_dev_mxfp4(layer, x, out, MODE_MFMA_FP8, ws)
+
+    if args.calib_copy_mib:
+        src = torch.ones(args.calib_copy_mib << 20, dtype=torch.uint8, device=hip.device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # warm up eagerly (also raises LDS limits, fills caches), then capture one step as a graph
     for _ in range(max(args.warmup, 2)):

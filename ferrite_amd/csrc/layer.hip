@@ -202,6 +202,8 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         PackedLayout L = packed_layout(s);
         rc = launch_router_chain(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), n, s.hidden,
                                  s.n_experts, logits, st);
+        if (rc == FERRITE_DECLINED)
+            rc = launch_matmul_exact(x, x_dtype, wts->router_w, nullptr, logits, n, s.hidden, s.n_experts, st);
     } else {
         rc = launch_matmul_exact(x, x_dtype, wts->router_w, nullptr, logits, n, s.hidden, s.n_experts, st);
     }

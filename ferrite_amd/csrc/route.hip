@@ -506,24 +506,20 @@ __global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const 
 
 // ------------------------------------------------------------------------------------------------
 // The head of the layer as ONE launch (decode-sized batches), or the router GEMM alone (kFused = false).
-//   blocks (eb, tb), eb < eblocks : router logits of tokens [4 tb, 4 tb + 4) (one per wave) for experts
-//                                   [64 eb, 64 eb + 64) (one per lane): the reference's sequential chain.  The
-//                                   router weight comes from its k-blocked transpose [H/4][Epad][4], so a
-//                                   128-k chunk of the block's 64 experts is one contiguous 32 KiB; chunks of
-//                                   it and of the four x rows are staged in LDS (two buffers) behind a
-//                                   two-chunk register prefetch, so the chains never wait on memory
-//   blocks (eblocks, tb)          : e4m3-per-32 quantisation of those four x rows (off the critical path)
-//   last logits wave of a token   : routes the token (arrival counter per token)
-//   last routed token             : builds the permutation and unit tables, then clears the counters so the
-//                                   next launch (or graph replay) starts clean
+// Every workgroup is a single wave.
+//   blocks (eb, t), eb < eblocks : router logits of token t for experts [64 eb, 64 eb + 64), one lane per
+//                                  expert: the reference's sequential chain.  The router weight comes from its
+//                                  k-blocked transpose [H/4][Epad][4], so the wave's load for four k is one
+//                                  contiguous 1 KiB; two register sets of 16 such loads alternate (the loads
+//                                  of one set fly while the chain consumes the other); x[t] sits in LDS as f32
+//   blocks (eblocks, t)          : e4m3-per-32 quantisation of x[t] (off the critical path)
+//   last logits wave of a token  : routes the token (arrival counter per token)
+//   last routed token            : builds the permutation and unit tables, then clears the counters so the
+//                                  next launch (or graph replay) starts clean
 // counters[0] = routed tokens, counters[1 + t] = logits blocks of token t that have arrived; all zero on entry.
 // ------------------------------------------------------------------------------------------------
 constexpr int HEAD_MAX_N = 256;
-constexpr int HD_TT = 4;          // tokens per block
-constexpr int HD_C4 = 32;         // float4 (4 k) per chunk and expert
-constexpr size_t HD_W_BYTES = (size_t)HD_C4 * 64 * 16;        // 32 KiB
-constexpr size_t HD_X_BYTES = (size_t)HD_TT * HD_C4 * 16;     // 2 KiB
-constexpr size_t HD_STAGE_BYTES = 2 * (HD_W_BYTES + HD_X_BYTES);
+constexpr int HD_D = 16;   // float4 loads per register set
 
 struct HeadArgs {
     const void* x;
@@ -538,127 +534,76 @@ struct HeadArgs {
     PermArgs perm;
 };
 
-struct HeadStage {
-    float4 w[8];
-    float4 x;
+struct HeadSet {
+    float4 w[HD_D];
 };
 
-template <typename XT>
-__device__ __forceinline__ void head_fetch(HeadStage& st, int c, int tid, const float4* __restrict__ wsrc, int Epad,
-                                           const XT* __restrict__ xrow) {
+__device__ __forceinline__ void head_load(HeadSet& st, const char* __restrict__ base, unsigned ldb, unsigned loff,
+                                          int k0, int nk4) {
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
-        const int i = tid + 256 * p;
-        st.w[p] = wsrc[(size_t)(c * HD_C4 + (i >> 6)) * Epad + (i & 63)];
-    }
-    const int k4 = c * HD_C4 + (tid & 31);   // threads >= 128 load a duplicate that is never stored
-    if constexpr (sizeof(XT) == 4) {
-        st.x = reinterpret_cast<const float4*>(xrow)[k4];
-    } else {
-        uint2 q = reinterpret_cast<const uint2*>(xrow)[k4];
-        st.x = make_float4(u2f(q.x << 16), u2f(q.x & 0xffff0000u), u2f(q.y << 16), u2f(q.y & 0xffff0000u));
+    for (int j = 0; j < HD_D; ++j) {
+        const int kn = min(k0 + j, nk4 - 1);   // past the end: a valid row that is never used
+        st.w[j] = *reinterpret_cast<const float4*>(base + (size_t)kn * ldb + loff);
     }
 }
 
-__device__ __forceinline__ void head_stash(const HeadStage& st, int buf, int tid, float4* w_lds, float4* x_lds) {
+__device__ __forceinline__ float head_chain(float s, const HeadSet& st, const float4* xl) {
 #pragma unroll
-    for (int p = 0; p < 8; ++p) w_lds[(size_t)buf * HD_C4 * 64 + tid + 256 * p] = st.w[p];
-    if (tid < HD_TT * HD_C4) x_lds[buf * HD_TT * HD_C4 + tid] = st.x;
-}
-
-// The chain over one staged chunk: 8 groups of 4 float4 in a rolled loop over pairs of groups with two named
-// register buffers, so that the LDS reads of a group are in flight while the previous group's 16 chain steps
-// execute (fully unrolled, the compiler hoists every read of the chunk and runs out of registers).
-__device__ __forceinline__ float head_chain(float s, const float4* wl, const float4* xl) {
-    constexpr int G = 4;
-    constexpr int NG = HD_C4 / G;
-    float4 wA[G], xA[G], wB[G], xB[G];
-#pragma unroll
-    for (int j = 0; j < G; ++j) { wA[j] = wl[j * 64]; xA[j] = xl[j]; }
-#pragma nounroll
-    for (int g = 0; g < NG; g += 2) {
-#pragma unroll
-        for (int j = 0; j < G; ++j) { wB[j] = wl[((g + 1) * G + j) * 64]; xB[j] = xl[(g + 1) * G + j]; }
-#pragma unroll
-        for (int j = 0; j < G; ++j) {
-            s = fadd(s, fmul(xA[j].x, wA[j].x));
-            s = fadd(s, fmul(xA[j].y, wA[j].y));
-            s = fadd(s, fmul(xA[j].z, wA[j].z));
-            s = fadd(s, fmul(xA[j].w, wA[j].w));
-        }
-        const int gn = g + 2 < NG ? g + 2 : NG - 1;   // the last pass re-reads a group it does not use
-#pragma unroll
-        for (int j = 0; j < G; ++j) { wA[j] = wl[(gn * G + j) * 64]; xA[j] = xl[gn * G + j]; }
-#pragma unroll
-        for (int j = 0; j < G; ++j) {
-            s = fadd(s, fmul(xB[j].x, wB[j].x));
-            s = fadd(s, fmul(xB[j].y, wB[j].y));
-            s = fadd(s, fmul(xB[j].z, wB[j].z));
-            s = fadd(s, fmul(xB[j].w, wB[j].w));
-        }
+    for (int j = 0; j < HD_D; ++j) {
+        const float4 xv = xl[j], wv = st.w[j];
+        s = fadd(s, fmul(xv.x, wv.x));
+        s = fadd(s, fmul(xv.y, wv.y));
+        s = fadd(s, fmul(xv.z, wv.z));
+        s = fadd(s, fmul(xv.w, wv.w));
     }
     return s;
 }
 
 template <typename XT, bool kFused>
-__global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
+__global__ __launch_bounds__(64) void moe_head_kernel(HeadArgs a) {
     extern __shared__ __align__(16) unsigned char head_lds[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int eb = blockIdx.x, t0 = blockIdx.y * HD_TT;
+    const int lane = threadIdx.x;
+    const int eb = blockIdx.x, t = blockIdx.y;
     const int eblocks = a.Epad >> 6;
     const int H = a.H;
-    const XT* xbase = static_cast<const XT*>(a.x);
+    const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
     if (eb == eblocks) {
-        const int bpr = H / 32;   // blocks per row
-        for (int i = tid; i < HD_TT * bpr; i += 256) {
-            const int t = t0 + i / bpr, b = i % bpr;
-            if (t < a.n)
-                a.xs[(size_t)t * bpr + b] = (uint8_t)quant_block32(xbase + (size_t)t * H + b * 32,
-                                                                   a.xq + (size_t)t * H + b * 32);
-        }
+        for (int b = lane; b < H / 32; b += 64)
+            a.xs[(size_t)t * (H / 32) + b] = (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
         return;
     }
-    float4* w_lds = reinterpret_cast<float4*>(head_lds);                      // [2][HD_C4][64]
-    float4* x_lds = reinterpret_cast<float4*>(head_lds + 2 * HD_W_BYTES);     // [2][HD_TT][HD_C4]
-    const int nk4 = H / 4;
-    const int nchunk = nk4 / HD_C4;
-    const float4* wsrc = reinterpret_cast<const float4*>(a.wt) + (size_t)eb * 64;
-
-    // H is a multiple of 128 here, so every chunk is full; rows past n are clamped to row n-1 (their results
-    // are never stored), which keeps the staging free of branches
-    const int xt = min(t0 + ((tid >> 5) & (HD_TT - 1)), a.n - 1);
-    const XT* xrow = xbase + (size_t)xt * H;
-    const float4* wl0 = w_lds + lane;
-    const float4* xl0 = x_lds + wave * HD_C4;
-    HeadStage sa, sb;
-    float s = 0.0f;
-    // The scheduling barriers pin the order "issue the loads of chunk c+2 -> chain over chunk c -> store chunk
-    // c+1 to LDS": without them the stores (and the wait for their global loads) drift in front of the chain.
-    head_fetch(sa, 0, tid, wsrc, a.Epad, xrow);
-    head_fetch(sb, nchunk > 1 ? 1 : 0, tid, wsrc, a.Epad, xrow);
-    head_stash(sa, 0, tid, w_lds, x_lds);
-    __syncthreads();
-    for (int c = 0; c < nchunk; c += 2) {
-        head_fetch(sa, min(c + 2, nchunk - 1), tid, wsrc, a.Epad, xrow);
-        __builtin_amdgcn_sched_barrier(0);
-        s = head_chain(s, wl0, xl0);
-        __builtin_amdgcn_sched_barrier(0);
-        head_stash(sb, 1, tid, w_lds, x_lds);
-        __syncthreads();
-        if (c + 1 < nchunk) {
-            head_fetch(sb, min(c + 3, nchunk - 1), tid, wsrc, a.Epad, xrow);
-            __builtin_amdgcn_sched_barrier(0);
-            s = head_chain(s, wl0 + (size_t)HD_C4 * 64, xl0 + HD_TT * HD_C4);
-            __builtin_amdgcn_sched_barrier(0);
-            head_stash(sa, 0, tid, w_lds, x_lds);
-            __syncthreads();
+    float4* xl = reinterpret_cast<float4*>(head_lds);
+    const int nk4 = H / 4;   // a multiple of 2 * HD_D (H % 128 == 0)
+    for (int i = lane; i < nk4; i += 64) {
+        float4 v;
+        if constexpr (sizeof(XT) == 4) {
+            v = reinterpret_cast<const float4*>(xrow)[i];
+        } else {
+            uint2 q = reinterpret_cast<const uint2*>(xrow)[i];
+            v = make_float4(u2f(q.x << 16), u2f(q.x & 0xffff0000u), u2f(q.y << 16), u2f(q.y & 0xffff0000u));
         }
+        xl[i] = v;
     }
-    const int t = t0 + wave, e = eb * 64 + lane;
-    const bool live = t < a.n;
-    if (live && e < a.E) a.logits[(size_t)t * a.E + e] = s;
+    const char* base = reinterpret_cast<const char*>(a.wt) + (size_t)eb * 64 * 16;
+    const unsigned ldb = (unsigned)a.Epad * 16, loff = (unsigned)lane * 16;
+    HeadSet sa, sb;
+    head_load(sa, base, ldb, loff, 0, nk4);
+    __syncthreads();
+    float s = 0.0f;
+    // the scheduling barriers pin "issue one set's loads, then chain over the other set"
+    for (int kk = 0; kk < nk4; kk += 2 * HD_D) {
+        head_load(sb, base, ldb, loff, kk + HD_D, nk4);
+        __builtin_amdgcn_sched_barrier(0);
+        s = head_chain(s, sa, xl + kk);
+        __builtin_amdgcn_sched_barrier(0);
+        head_load(sa, base, ldb, loff, kk + 2 * HD_D, nk4);
+        __builtin_amdgcn_sched_barrier(0);
+        s = head_chain(s, sb, xl + kk + HD_D);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    const int e = eb * 64 + lane;
+    if (e < a.E) a.logits[(size_t)t * a.E + e] = s;
     if constexpr (!kFused) return;
-    if (!live) return;   // wave-uniform; no block-wide barrier follows
 
     // arrival: the stores above are made visible before the counter moves
     __threadfence();
@@ -667,8 +612,8 @@ __global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
     last = __shfl(last, 0, 64);
     if (!last) return;
     __threadfence();
-    // the staging buffers are dead for this wave; each wave takes a private slice of them as scratch
-    RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds + (size_t)wave * sizeof(RouteScratch));
+    __syncthreads();   // x in LDS is dead from here; the scratch below aliases it
+    RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds);
     route_wave<true>(a.logits + (size_t)t * a.E, a.bias, true, a.E, a.topk, a.n_group, a.topk_group, a.scaling, sc,
                      a.probs + (size_t)t * a.topk, a.ids_f32 + (size_t)t * a.topk, a.ids + (size_t)t * a.topk);
     __threadfence();
@@ -677,40 +622,28 @@ __global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
     last = __shfl(last, 0, 64);
     if (!last) return;
     __threadfence();
-    // the permutation scratch sits above the four routing scratches (another wave may still be routing)
-    permute_in_block<true, true>(a.perm, reinterpret_cast<unsigned long long*>(head_lds + 4 * sizeof(RouteScratch)));
+    __syncthreads();
+    permute_in_block<true, true>(a.perm, reinterpret_cast<unsigned long long*>(head_lds));
     for (int i = lane; i < a.n + 1; i += 64) a.counters[i] = 0;
 }
 
-static size_t head_lds_bytes(int n, int E, bool fused) {
-    size_t b = HD_STAGE_BYTES;
+static size_t head_lds_bytes(int n, int H, int E, bool fused) {
+    size_t b = (size_t)H * 4;
     if (fused) {
-        size_t p = 4 * sizeof(RouteScratch) + perm_block_lds_bytes(n, E);
+        if (b < sizeof(RouteScratch)) b = sizeof(RouteScratch);
+        size_t p = perm_block_lds_bytes(n, E);
         if (p > b) b = p;
     }
     return b;
 }
 
 bool head_supported(int n, int H, int E) {
-    return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, E, true) <= 150 * 1024;
-}
-
-template <typename K>
-static int raise_lds(K kernel, size_t bytes, size_t* raised) {
-    if (bytes <= 64 * 1024 || bytes <= *raised) return FERRITE_OK;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-    *raised = bytes;
-    return FERRITE_OK;
+    return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, H, E, true) <= 60 * 1024;
 }
 
 template <typename XT, bool kFused>
 static int launch_head_t(const HeadArgs& a, dim3 grid, size_t lds, hipStream_t st) {
-    static size_t raised = 0;
-    int rc = raise_lds(moe_head_kernel<XT, kFused>, lds, &raised);
-    if (rc) return rc;
-    moe_head_kernel<XT, kFused><<<grid, 256, lds, st>>>(a);
+    moe_head_kernel<XT, kFused><<<grid, 64, lds, st>>>(a);
     return check_launch("moe_head");
 }
 
@@ -733,8 +666,8 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
         p.unit_expert = units->unit_expert; p.unit_row0 = units->unit_row0; p.unit_rows = units->unit_rows;
         p.n_units = units->n_units; p.unit_cap = units->unit_rows_cap; p.max_units = units->max_units;
     }
-    dim3 grid(a.Epad / 64 + (xq ? 1 : 0), (n + HD_TT - 1) / HD_TT);
-    const size_t lds = head_lds_bytes(n, s.n_experts, true);
+    dim3 grid(a.Epad / 64 + (xq ? 1 : 0), n);
+    const size_t lds = head_lds_bytes(n, s.hidden, s.n_experts, true);
     if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, grid, lds, st);
     if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, true>(a, grid, lds, st);
     return FERRITE_ERR_INVALID_ARG;
@@ -743,11 +676,11 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
 // Router GEMM alone from the transposed weight (any n): logits only.
 int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
                         hipStream_t st) {
-    if (H % 128 != 0 || n <= 0) return FERRITE_DECLINED;
+    if (H % 128 != 0 || n <= 0 || (size_t)H * 4 > 60 * 1024 || n > 65535) return FERRITE_DECLINED;
     HeadArgs a{};
     a.x = x; a.wt = router_t; a.n = n; a.H = H; a.E = E; a.Epad = (E + 63) / 64 * 64; a.logits = logits;
-    dim3 grid(a.Epad / 64, (n + HD_TT - 1) / HD_TT);
-    const size_t lds = head_lds_bytes(n, E, false);
+    dim3 grid(a.Epad / 64, n);
+    const size_t lds = head_lds_bytes(n, H, E, false);
     if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, false>(a, grid, lds, st);
     if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, false>(a, grid, lds, st);
     return FERRITE_ERR_INVALID_ARG;
