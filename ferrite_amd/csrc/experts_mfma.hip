@@ -113,41 +113,49 @@ __device__ __forceinline__ void mfma_step(const u4v (&a)[4], const u4v& sc, cons
     }
 }
 
-__device__ __forceinline__ void stream_item(const u4v* __restrict__ wp, const u4v* __restrict__ sp, int KT,
-                                            const u4v* bq, const uint32_t* bsc, int lane, v4f (&acc)[4]) {
-    const int KT4 = (KT + 3) >> 2;
+// Registers of the weight stream: two buffers of one group (4 k steps x 4 tiles) each.
+struct StreamRegs {
     u4v a[2][4][4];   // [buffer][k step in group][tile]
     u4v sc[2];
-    auto load_group = [&](int g4, int buf) {
-        sc[buf] = __builtin_nontemporal_load(&sp[(size_t)g4 * 64 + lane]);
+};
+
+__device__ __forceinline__ void stream_load_group(StreamRegs& r, const u4v* __restrict__ wp,
+                                                  const u4v* __restrict__ sp, int KT, int lane, int g4, int buf) {
+    r.sc[buf] = __builtin_nontemporal_load(&sp[(size_t)g4 * 64 + lane]);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int kt = g4 * 4 + q;
-            if (kt < KT) {
+    for (int q = 0; q < 4; ++q) {
+        const int kt = g4 * 4 + q;
+        if (kt < KT) {
 #pragma unroll
-                for (int t = 0; t < 4; ++t) a[buf][q][t] = __builtin_nontemporal_load(&wp[((size_t)kt * 4 + t) * 64 + lane]);
-            }
+            for (int t = 0; t < 4; ++t)
+                r.a[buf][q][t] = __builtin_nontemporal_load(&wp[((size_t)kt * 4 + t) * 64 + lane]);
         }
-    };
-    load_group(0, 0);
+    }
+}
+
+// The item's group 0 must already be in flight in buffer 0 (stream_load_group(..., 0, 0)): callers issue it
+// before they fill LDS, so the first weights travel while the activations are staged.
+__device__ __forceinline__ void stream_item(StreamRegs& r, const u4v* __restrict__ wp, const u4v* __restrict__ sp,
+                                            int KT, const u4v* bq, const uint32_t* bsc, int lane, v4f (&acc)[4]) {
+    const int KT4 = (KT + 3) >> 2;
     for (int g4 = 0; g4 < KT4; g4 += 2) {
-        if (g4 + 1 < KT4) load_group(g4 + 1, 1);
+        if (g4 + 1 < KT4) stream_load_group(r, wp, sp, KT, lane, g4 + 1, 1);
         {
             const uint32_t bs = bsc[g4 * 64 + lane];
             const int kt = g4 * 4;
-            mfma_step<0>(a[0][0], sc[0], bq, bs, kt, lane, acc);
-            if (kt + 1 < KT) mfma_step<1>(a[0][1], sc[0], bq, bs, kt + 1, lane, acc);
-            if (kt + 2 < KT) mfma_step<2>(a[0][2], sc[0], bq, bs, kt + 2, lane, acc);
-            if (kt + 3 < KT) mfma_step<3>(a[0][3], sc[0], bq, bs, kt + 3, lane, acc);
+            mfma_step<0>(r.a[0][0], r.sc[0], bq, bs, kt, lane, acc);
+            if (kt + 1 < KT) mfma_step<1>(r.a[0][1], r.sc[0], bq, bs, kt + 1, lane, acc);
+            if (kt + 2 < KT) mfma_step<2>(r.a[0][2], r.sc[0], bq, bs, kt + 2, lane, acc);
+            if (kt + 3 < KT) mfma_step<3>(r.a[0][3], r.sc[0], bq, bs, kt + 3, lane, acc);
         }
         if (g4 + 1 < KT4) {
-            if (g4 + 2 < KT4) load_group(g4 + 2, 0);
+            if (g4 + 2 < KT4) stream_load_group(r, wp, sp, KT, lane, g4 + 2, 0);
             const uint32_t bs = bsc[(g4 + 1) * 64 + lane];
             const int kt = (g4 + 1) * 4;
-            mfma_step<0>(a[1][0], sc[1], bq, bs, kt, lane, acc);
-            if (kt + 1 < KT) mfma_step<1>(a[1][1], sc[1], bq, bs, kt + 1, lane, acc);
-            if (kt + 2 < KT) mfma_step<2>(a[1][2], sc[1], bq, bs, kt + 2, lane, acc);
-            if (kt + 3 < KT) mfma_step<3>(a[1][3], sc[1], bq, bs, kt + 3, lane, acc);
+            mfma_step<0>(r.a[1][0], r.sc[1], bq, bs, kt, lane, acc);
+            if (kt + 1 < KT) mfma_step<1>(r.a[1][1], r.sc[1], bq, bs, kt + 1, lane, acc);
+            if (kt + 2 < KT) mfma_step<2>(r.a[1][2], r.sc[1], bq, bs, kt + 2, lane, acc);
+            if (kt + 3 < KT) mfma_step<3>(r.a[1][3], r.sc[1], bq, bs, kt + 3, lane, acc);
         }
     }
 }
@@ -232,20 +240,22 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
         int i = gather_src[g];
         return (i < 0 || i >= nk) ? -1 : i / topk;
     };
-    fill_b_operand(xq, xs, H, nrows, row_src, bq, bsc);
-    __syncthreads();
-
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int item = blockIdx.x * WAVES + wave;
-    if (item >= items) return;
+    const bool live = item < items;
     const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
     const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
     const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
     const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
+    StreamRegs regs;
+    if (live) stream_load_group(regs, wp, sp, KT, lane, 0, 0);   // weights fly while the activations are staged
+    fill_b_operand(xq, xs, H, nrows, row_src, bq, bsc);
+    __syncthreads();
+    if (!live) return;
     v4f acc[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-    stream_item(wp, sp, KT, bq, bsc, lane, acc);
+    stream_item(regs, wp, sp, KT, bq, bsc, lane, acc);
 
     // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
     float r0[4], r1[4];
@@ -291,6 +301,15 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
     const int KT = inter / 128, KT4 = (KT + 3) / 4;
     u4v* bq = reinterpret_cast<u4v*>(lds_raw);
     uint32_t* bsc = reinterpret_cast<uint32_t*>(lds_raw + (size_t)a.act_ld * 16);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int item0 = (blockIdx.x * WAVES + wave) * IPW;
+    StreamRegs regs;
+    if (item0 < items) {   // the first item's weights fly while the activations are staged
+        const uint8_t* cb = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
+        const uint8_t* sb = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
+        stream_load_group(regs, reinterpret_cast<const u4v*>(cb) + (size_t)item0 * KT * 256,
+                          reinterpret_cast<const u4v*>(sb) + (size_t)item0 * KT4 * 64, KT, lane, 0, 0);
+    }
     // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
     {
         const int chunks = inter / 16;
@@ -315,20 +334,20 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
         }
     }
     __syncthreads();
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
     const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
     const int c = lane & 15, g = lane >> 4;
 #pragma unroll 1
     for (int ii = 0; ii < IPW; ++ii) {
-        const int item = (blockIdx.x * WAVES + wave) * IPW + ii;
+        const int item = item0 + ii;
         if (item >= items) break;
         const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
         const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
+        if (ii > 0) stream_load_group(regs, wp, sp, KT, lane, 0, 0);
         v4f acc[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-        stream_item(wp, sp, KT, bq, bsc, lane, acc);
+        stream_item(regs, wp, sp, KT, bq, bsc, lane, acc);
         if (c < nrows) {
             float* dst = y + (size_t)(row0 + c) * H + (size_t)item * 64 + g * 4;
 #pragma unroll
