@@ -26,6 +26,11 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 MFMA_PEAK_FP8_TFLOPS = 5000.0  # dense fp8-operand MFMA (e4m3 activations x e2m1 weights run at this rate)
 MFMA_PEAK_FP4_TFLOPS = 10100.0 # dense MXFP4 x MXFP4
 
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
+# counters' reading for a 1 GiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw values
+# are in profiles/c1_decode32_hbm_counters.md.  Counters cannot be read inside this script.
+MEASURED_TRAFFIC = {("c1", "gate_up_mfma_kernel"): 770.6e6}
+
 WORKLOADS = {
     "c0": "c0: tiny parity layer, 8 tokens, H256 E16 top4 (4 groups/2) I128, MXFP4 weights, f32 activations",
     "c1": "c1: GLM-5.3-Flash-shaped decode MoE layer, 32 tokens, H4096 E128+1 shared top8 (8 groups/4) I1536, "
@@ -177,10 +182,8 @@ def main():
     roofline = {"bound": "hbm", "kernel": "gate_up_mfma_kernel", "achieved": round(gate_up_gbs, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gate_up_gbs / HBM_PEAK_GBS, 4), "traffic": None,
                 "algorithmic_bytes_per_launch": ab["gate_up"], "avg_launch_us": round(stage_us["gate_up_mfma"], 2)}
-    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(traffic_file):
-        with open(traffic_file) as f:
-            roofline["traffic"] = json.load(f).get(f"gate_up_mfma_kernel:{args.config}")
+    if not args.tokens:
+        roofline["traffic"] = MEASURED_TRAFFIC.get((args.config, "gate_up_mfma_kernel"))
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -194,7 +197,7 @@ def main():
         while True:
             oracle.moe_ffn_mxfp4(inp, act_mode=0, n_threads=1, tok_sel=sel)
             reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 4:
+            if time.perf_counter() - t0 > 12.0 or reps >= 12:
                 break
         t1 = (time.perf_counter() - t0) / reps
         ncores = min(16, os.cpu_count() or 1)
