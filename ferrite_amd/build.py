@@ -53,5 +53,25 @@ def build(verbose: bool = False) -> str:
     return SO_PATH
 
 
+HOST_DIR = os.path.join(HERE, "host")
+HOST_SMOKE = os.path.join(HOST_DIR, "hip_backend_smoke")
+
+
+def build_host(verbose: bool = False) -> str:
+    """Compile the C++ host side (HipBackend over the C ABI) and its smoke driver with g++."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", "-o", HOST_SMOKE,
+           os.path.join(HOST_DIR, "hip_backend.cpp"), os.path.join(HOST_DIR, "smoke_main.cpp"),
+           f"-L{rocm}/lib", "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm}/lib"]
+    if verbose:
+        print(" ".join(cmd))
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+        raise RuntimeError("g++ failed (host side)")
+    return HOST_SMOKE
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_host(verbose=True))

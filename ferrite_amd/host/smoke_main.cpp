@@ -1,0 +1,210 @@
+// GPU smoke tests of the C++ HipBackend, written like the reference's own tests: the golden values of
+// crates/ferrite-kernel/tests/golden.rs (matmul, swiglu, moe_route) and the fused-MoE parity test of
+// crates/ferrite-kernel/tests/gpu_smoke.rs:429-601 (its fixture, its in-test CPU reference, its tolerance),
+// plus a capture/replay check (gpu_smoke.rs:268-306).  Usage: hip_backend_smoke <path to libferrite_hip.so>
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <numeric>
+
+#include "hip_backend.hpp"
+
+using namespace ferrite;
+
+static int failures = 0;
+#define CHECK(cond, ...)                                   \
+    do {                                                   \
+        if (!(cond)) { ++failures; std::printf("FAIL %s:%d: ", __FILE__, __LINE__); std::printf(__VA_ARGS__); std::printf("\n"); } \
+    } while (0)
+
+static Tensor t2(size_t r, size_t c, std::vector<float> v) { return Tensor::from_f32({r, c}, std::move(v)); }
+
+static void matmul_matches_manual(HipBackend& b) {   // golden.rs:14-27
+    Tensor x = t2(2, 2, {1, 2, 3, 4}), w = t2(2, 2, {5, 6, 7, 8}), out = Tensor::zeros({2, 2});
+    b.matmul(x, w, nullptr, out);
+    CHECK(out.data == std::vector<float>({17, 23, 39, 53}), "matmul");
+    Tensor bias = t2(1, 2, {0.5f, -0.5f});
+    b.matmul(x, w, &bias, out);
+    CHECK(out.data == std::vector<float>({17.5f, 22.5f, 39.5f, 52.5f}), "matmul+bias");
+    bool threw = false;
+    try { Tensor w3 = Tensor::zeros({2, 3}); b.matmul(x, w3, nullptr, out); } catch (const FerriteError& e) { threw = e.kind == FerriteError::ShapeMismatch; }
+    CHECK(threw, "k mismatch must be ShapeMismatch");
+    threw = false;
+    try { Tensor o3 = Tensor::zeros({3, 2}); b.matmul(x, w, nullptr, o3); } catch (const FerriteError& e) { threw = e.kind == FerriteError::InvalidArg; }
+    CHECK(threw, "bad out shape must be InvalidArg");
+}
+
+static void swiglu_clamps(HipBackend& b) {   // golden.rs:44-55
+    Tensor gu = t2(1, 4, {2, 20, 3, 1}), out = Tensor::zeros({1, 2});
+    b.swiglu_limited(gu, 10.0f, out);
+    float silu2 = 2.0f / (1.0f + std::exp(-2.0f));
+    CHECK(std::fabs(out.data[0] - silu2 * 3.0f) < 1e-6f, "swiglu[0]");
+    CHECK(std::fabs(out.data[1] - 10.0f / (1.0f + std::exp(-10.0f))) < 1e-6f, "gate clamped to 10");
+}
+
+static void moe_route_noaux_tc(HipBackend& b) {   // golden.rs:189-210 and gpu_smoke.rs:139-155
+    Tensor logits = t2(1, 3, {1.0f, 2.0f, 0.5f}), bias = t2(1, 3, {0, 0, 0.5f});
+    Tensor probs = Tensor::zeros({1, 2}), ids = Tensor::zeros({1, 2});
+    b.moe_route(logits, bias, 2, 1.0f, probs, ids);
+    float s1 = 1.0f / (1.0f + std::exp(-2.0f)), s2 = 1.0f / (1.0f + std::exp(-0.5f));
+    CHECK(ids.data[0] == 2.0f && ids.data[1] == 1.0f, "ids %g %g", ids.data[0], ids.data[1]);
+    CHECK(std::fabs(probs.data[0] - s2 / (s1 + s2)) < 1e-5f && std::fabs(probs.data[1] - s1 / (s1 + s2)) < 1e-5f, "probs");
+    // the tie-free ramp of the reference's GPU test: n=2, e=288, topk=8, scale 2.5
+    const size_t n = 2, e = 288, k = 8;
+    std::vector<float> lg(n * e), bs(e);
+    for (size_t i = 0; i < n * e; ++i) lg[i] = (float)i * 0.017f - 2.0f;
+    for (size_t i = 0; i < e; ++i) bs[i] = (float)(i % 11) * 0.01f;
+    Tensor L = t2(n, e, lg), B = Tensor::from_f32({e}, bs), P = Tensor::zeros({n, k}), I = Tensor::zeros({n, k});
+    b.moe_route(L, B, k, 2.5f, P, I);
+    for (size_t r = 0; r < n; ++r) {   // CpuBackend::moe_route restated (cpu.rs:546-569)
+        std::vector<float> sig(e);
+        std::vector<size_t> order(e);
+        for (size_t j = 0; j < e; ++j) { sig[j] = 1.0f / (1.0f + std::exp(-lg[r * e + j])); order[j] = j; }
+        std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t c) { return sig[a] + bs[a] > sig[c] + bs[c]; });
+        float sum = 0;
+        for (size_t q = 0; q < k; ++q) sum += sig[order[q]];
+        for (size_t q = 0; q < k; ++q) {
+            CHECK(I.data[r * k + q] == (float)order[q], "ramp ids row %zu slot %zu", r, q);
+            CHECK(std::fabs(P.data[r * k + q] - sig[order[q]] / (sum + 1.1920929e-7f) * 2.5f) < 1e-5f, "ramp probs");
+        }
+    }
+}
+
+// ---- the fused MoE fixture of gpu_smoke.rs:437-470 ----
+static float bex(size_t i, size_t s) { return (float)((i + s) % 4) * 0.25f - 0.5f; }
+// encode a matrix with values in {-0.5,-0.25,0,0.25} as MXFP4 with scale 2^-2 (byte 125): value = code * 0.25
+static void encode(const std::vector<float>& m, size_t rows, size_t cols, std::vector<uint8_t>& codes, std::vector<uint8_t>& scales) {
+    codes.assign(rows * cols / 2, 0);
+    scales.assign(rows * cols / 32, 125);
+    for (size_t i = 0; i < rows * cols; ++i) {
+        float q = m[i] * 4.0f;   // -2, -1, 0, 1
+        uint8_t c = q == 0 ? 0 : (q == 1 ? 2 : (q == -1 ? 10 : 12));
+        codes[i / 2] |= (i % 2) ? (uint8_t)(c << 4) : c;
+    }
+}
+
+static void moe_fused_parity(HipBackend& b) {
+    const size_t H = 64, I = 32, Is = 16, IsP = 32, E = 8, K = 2;
+    const float scaling = 1.2f, limit = 7.0f;
+    std::vector<float> x(H), gate_w(E * H), bias(E);
+    for (size_t i = 0; i < H; ++i) x[i] = bex(i, 0);
+    for (size_t i = 0; i < E * H; ++i) gate_w[i] = bex(i, 5);
+    for (size_t i = 0; i < E; ++i) bias[i] = bex(i, 2);
+    auto mk = [](size_t r, size_t c, size_t s) { std::vector<float> v(r * c); for (size_t i = 0; i < r * c; ++i) v[i] = bex(i * 7 + s, 0); return v; };
+    std::vector<std::vector<float>> eg, eu, ed;
+    for (size_t s = 0; s < E; ++s) { eg.push_back(mk(I, H, s * 11)); eu.push_back(mk(I, H, s * 13 + 3)); ed.push_back(mk(H, I, s * 17 + 7)); }
+    std::vector<float> sg = mk(Is, H, 29), su = mk(Is, H, 31), sd = mk(H, Is, 37);
+    // stack experts; pad the 16-wide shared expert to one 32-wide MXFP4 block with zeros (an exact no-op)
+    std::vector<float> G(E * I * H), U(E * I * H), D(E * H * I), SG(IsP * H, 0.f), SU(IsP * H, 0.f), SD(H * IsP, 0.f);
+    for (size_t e = 0; e < E; ++e) {
+        std::copy(eg[e].begin(), eg[e].end(), G.begin() + e * I * H);
+        std::copy(eu[e].begin(), eu[e].end(), U.begin() + e * I * H);
+        std::copy(ed[e].begin(), ed[e].end(), D.begin() + e * H * I);
+    }
+    std::copy(sg.begin(), sg.end(), SG.begin());
+    std::copy(su.begin(), su.end(), SU.begin());
+    for (size_t h = 0; h < H; ++h) for (size_t i = 0; i < Is; ++i) SD[h * IsP + i] = sd[h * Is + i];
+    std::vector<uint8_t> gw, gs, uw, us, dw, ds, sgw, sgs, suw, sus, sdw, sds;
+    encode(G, E * I, H, gw, gs); encode(U, E * I, H, uw, us); encode(D, E * H, I, dw, ds);
+    encode(SG, IsP, H, sgw, sgs); encode(SU, IsP, H, suw, sus); encode(SD, H, IsP, sdw, sds);
+    ferrite_moe_shape shape{(int)H, (int)E, (int)K, (int)I, (int)IsP, 1, 1, scaling, limit};
+    MoeHostWeights hw{gate_w.data(), bias.data(), gw.data(), gs.data(), uw.data(), us.data(), dw.data(), ds.data(),
+                      sgw.data(), sgs.data(), suw.data(), sus.data(), sdw.data(), sds.data()};
+    MoeLayerDev layer = b.load_moe_layer(shape, hw);
+    DevBuf dx(H * 4), dout(H * 4);
+    dx.upload(x.data(), H * 4);
+    b.moe_layer_dev_mxfp4(layer, dx, FERRITE_DT_F32, 1, dout, FERRITE_DT_F32, FERRITE_MODE_F32_CHECK);
+    b.sync();
+    std::vector<float> hv(H);
+    dout.download(hv.data(), H * 4);
+
+    // CPU reference spelled out as in gpu_smoke.rs:493-562
+    std::vector<float> logits(E), scores(E), choice(E);
+    for (size_t j = 0; j < E; ++j) { float s = 0; for (size_t k = 0; k < H; ++k) s += x[k] * gate_w[j * H + k]; logits[j] = s; }
+    for (size_t j = 0; j < E; ++j) { scores[j] = 1.0f / (1.0f + std::exp(-logits[j])); choice[j] = scores[j] + bias[j]; }
+    std::vector<size_t> order(E);
+    std::iota(order.begin(), order.end(), 0);
+    std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t c) { return choice[a] > choice[c]; });
+    float rsum = scores[order[0]] + scores[order[1]];
+    auto silu = [](float g) { return g / (1.0f + std::exp(-g)); };
+    std::vector<float> ref(H, 0.f);
+    auto run_expert = [&](const std::vector<float>& g, const std::vector<float>& u, const std::vector<float>& d, size_t inter, float wgt) {
+        std::vector<float> act(inter);
+        for (size_t i = 0; i < inter; ++i) {
+            float gv = 0, uv = 0;
+            for (size_t k = 0; k < H; ++k) { gv += x[k] * g[i * H + k]; uv += x[k] * u[i * H + k]; }
+            gv = std::fmin(gv, limit);
+            uv = std::fmin(std::fmax(uv, -limit), limit);
+            act[i] = silu(gv) * uv;
+        }
+        for (size_t h = 0; h < H; ++h) { float y = 0; for (size_t i = 0; i < inter; ++i) y += act[i] * d[h * inter + i]; ref[h] += wgt * y; }
+    };
+    for (size_t jj = 0; jj < K; ++jj) run_expert(eg[order[jj]], eu[order[jj]], ed[order[jj]], I, scores[order[jj]] / rsum * scaling);
+    run_expert(sg, su, sd, Is, 1.0f);
+    float maxd = 0;
+    for (size_t i = 0; i < H; ++i) maxd = std::fmax(maxd, std::fabs(hv[i] - ref[i]));
+    CHECK(maxd < 1e-4f, "moe_fused mismatch: max diff %g (tol 1e-4)", maxd);
+    std::printf("[moe-fused] parity max_diff %g (ids %zu %zu)\n", maxd, order[0], order[1]);
+}
+
+static void graph_capture_smoke(HipBackend& b) {   // gpu_smoke.rs:268-306: capture, replay, same result as eager
+    const int H = 256, I = 128, E = 8, K = 2, n = 24;
+    ferrite_moe_shape shape{H, E, K, I, I, 4, 2, 2.5f, 10.0f};
+    uint64_t st = 0x9E3779B97F4A7C15ull;
+    auto rnd = [&]() { st ^= st >> 12; st ^= st << 25; st ^= st >> 27; return st * 0x2545F4914F6CDD1Dull; };   // xorshift64*
+    auto bytes = [&](size_t nb) { std::vector<uint8_t> v(nb); for (auto& c : v) c = (uint8_t)(rnd() >> 56); return v; };
+    auto scl = [&](size_t nb) { std::vector<uint8_t> v(nb); for (auto& c : v) c = 119 + (uint8_t)((rnd() >> 60) & 1); return v; };
+    std::vector<float> rw((size_t)E * H), rb(E);
+    for (auto& v : rw) v = ((float)(rnd() >> 40) / 16777216.0f - 0.5f) * 0.1f;
+    for (auto& v : rb) v = ((float)(rnd() >> 40) / 16777216.0f - 0.5f) * 0.02f;
+    auto gw = bytes((size_t)E * I * H / 2), uw = bytes((size_t)E * I * H / 2), dw = bytes((size_t)E * H * I / 2);
+    auto gs = scl((size_t)E * I * H / 32), us = scl((size_t)E * I * H / 32), ds = scl((size_t)E * H * I / 32);
+    auto sgw = bytes((size_t)I * H / 2), suw = bytes((size_t)I * H / 2), sdw = bytes((size_t)H * I / 2);
+    auto sgs = scl((size_t)I * H / 32), sus = scl((size_t)I * H / 32), sds = scl((size_t)H * I / 32);
+    MoeHostWeights hw{rw.data(), rb.data(), gw.data(), gs.data(), uw.data(), us.data(), dw.data(), ds.data(),
+                      sgw.data(), sgs.data(), suw.data(), sus.data(), sdw.data(), sds.data()};
+    MoeLayerDev layer = b.load_moe_layer(shape, hw);
+    DevBuf dx((size_t)n * H * 4), dout((size_t)n * H * 4), deager((size_t)n * H * 4);
+    std::vector<float> x((size_t)n * H);
+    auto fill = [&]() { for (auto& v : x) v = ((float)(rnd() >> 40) / 16777216.0f - 0.5f) * 4.0f; };
+    fill();
+    dx.upload(x.data(), x.size() * 4);
+    b.moe_layer_dev_mxfp4(layer, dx, FERRITE_DT_F32, n, dout, FERRITE_DT_F32, FERRITE_MODE_MFMA_FP8);   // warm
+    b.sync();
+    b.begin_capture();
+    b.moe_layer_dev_mxfp4(layer, dx, FERRITE_DT_F32, n, dout, FERRITE_DT_F32, FERRITE_MODE_MFMA_FP8);
+    OpTrace trace = b.end_capture();
+    CHECK(trace.len() == 1 && trace.ops[0].op == "moe_layer_mxfp4", "trace ops");
+    std::vector<float> a((size_t)n * H), c((size_t)n * H);
+    for (int rep = 0; rep < 3; ++rep) {
+        fill();
+        dx.upload(x.data(), x.size() * 4);
+        b.moe_layer_dev_mxfp4(layer, dx, FERRITE_DT_F32, n, deager, FERRITE_DT_F32, FERRITE_MODE_MFMA_FP8);
+        b.sync();
+        b.begin_verify(trace);
+        CHECK(b.end_verify(), "replay failed");
+        dout.download(a.data(), a.size() * 4);
+        deager.download(c.data(), c.size() * 4);
+        CHECK(std::memcmp(a.data(), c.data(), a.size() * 4) == 0, "replay %d differs from eager", rep);
+    }
+    b.graph_destroy(trace);
+}
+
+int main(int argc, char** argv) {
+    if (argc < 2) { std::printf("usage: %s libferrite_hip.so\n", argv[0]); return 2; }
+    try {
+        HipBackend b(argv[1], 0);
+        std::printf("build id %s\n", b.build_id().c_str());
+        matmul_matches_manual(b); std::printf("matmul ok\n"); std::fflush(stdout);
+        swiglu_clamps(b); std::printf("swiglu ok\n"); std::fflush(stdout);
+        moe_route_noaux_tc(b); std::printf("moe_route ok\n"); std::fflush(stdout);
+        moe_fused_parity(b); std::fflush(stdout);
+        graph_capture_smoke(b); std::printf("graph ok\n");
+    } catch (const std::exception& e) {
+        std::printf("EXCEPTION: %s\n", e.what());
+        return 1;
+    }
+    std::printf(failures ? "FAILED (%d)\n" : "ALL OK\n", failures);
+    return failures ? 1 : 0;
+}

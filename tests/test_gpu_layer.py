@@ -162,3 +162,14 @@ def test_layer_repeated_calls_same_workspace(hip, oracle):
         first = out if first is None else first
         assert np.array_equal(out, first)
     assert max_abs_rel(first, ref["out"]) <= TOL_MFMA
+
+
+def test_cpp_host_backend_smoke():
+    """The C++ HipBackend (ferrite_amd/host) over the same C ABI: golden.rs values, the gpu_smoke.rs fused-MoE
+    fixture against its in-test CPU reference, and capture/replay.  One child process."""
+    import subprocess
+    from ferrite_amd import build as hip_build
+    assert os.path.exists(hip_build.HOST_SMOKE), "build the host side first: python -m ferrite_amd.build"
+    res = subprocess.run([hip_build.HOST_SMOKE, hip_build.SO_PATH], capture_output=True, text=True, timeout=120)
+    print(res.stdout[-2000:], res.stderr[-2000:])
+    assert res.returncode == 0 and "ALL OK" in res.stdout
