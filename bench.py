@@ -36,6 +36,7 @@ WORKLOADS = {
     "c1": "c1: GLM-5.3-Flash-shaped decode MoE layer, 32 tokens, H4096 E128+1 shared top8 (8 groups/4) I1536, "
           "MXFP4 weights, bf16 activations",
     "c2": "c2: same layer at prefill chunk, 4096 tokens, e4m3/32 activations",
+    "c3": "c3: DeepSeek-V3-scale skewed layer, 8192 tokens, H7168 E256+1 top8 (8 groups/4) I2048, Zipf(1.1) bias",
     "c4": "c4: 42-MoE-layer decode step of the GLM-5.3-Flash shape at 192 tokens (batch 64 x MTP 3), all layers in one "
           "hipGraph; every layer has its own weights (54 GB resident) and reads the same static 192-token input",
 }
@@ -231,6 +232,7 @@ def main():
         "us_per_layer": round(us_layer, 2), "us_per_layer_eager_events": round(eager_us, 2),
         "stage_us": {k: round(v, 2) for k, v in stage_us.items()},
         "experts_hit": n_active, "max_tokens_per_expert": int(counts.max()),
+        "max_over_mean_tokens_per_expert": round(float(counts.max() / max(counts.mean(), 1e-9)), 2),
         "layer_algorithmic_bytes": ab["total"],
         "layer_hbm_gbs": round(ab["total"] / (us_layer * 1e-6) / 1e9, 1),
         "layer_hbm_frac": round(ab["total"] / (us_layer * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),

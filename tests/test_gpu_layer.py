@@ -173,3 +173,44 @@ def test_cpp_host_backend_smoke():
     res = subprocess.run([hip_build.HOST_SMOKE, hip_build.SO_PATH], capture_output=True, text=True, timeout=120)
     print(res.stdout[-2000:], res.stderr[-2000:])
     assert res.returncode == 0 and "ALL OK" in res.stdout
+
+
+def _scale_check(hip, oracle, cfg, n_sample, seed=0):
+    """Full-size run: routing and permutation bit-exact for every token, layer output against the oracle on a
+    token sample, and a size-independent property: the layer is a per-token function, so permuting the tokens
+    permutes the output rows bit for bit."""
+    inp = synth.make_inputs(cfg, seed=seed)
+    layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
+    out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8, bf16=cfg.act_bf16)
+    ref = oracle.moe_ffn_mxfp4(inp, n_threads=16, want_out=False)
+    check_routing(v, ref, oracle, cfg)
+    sel = np.linspace(0, cfg.n - 1, n_sample).astype(np.int32)
+    sub = oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=16, tok_sel=sel)
+    err = max_abs_rel(out[sel], sub["out"])
+    counts = v["counts"]
+    print(f"{cfg.name}: sample err {err:.3e}; tokens/expert max {counts.max()} mean {counts.mean():.1f}; "
+          f"experts hit {(counts > 0).sum()}")
+    assert err <= TOL_MFMA
+    perm = np.random.default_rng(1).permutation(cfg.n)
+    out_p, _ = run_layer(hip, layer, inp.x[perm], MODE_MFMA_FP8, bf16=cfg.act_bf16)
+    assert np.array_equal(out_p, out[perm])
+    return v
+
+
+def test_layer_c2_prefill_scale(hip, oracle):
+    """4096 tokens, ~256 tokens per expert."""
+    _scale_check(hip, oracle, synth.CONFIGS["c2"], n_sample=12)
+
+
+def test_layer_c4_decode192(hip, oracle):
+    _scale_check(hip, oracle, synth.CONFIGS["c4"], n_sample=12)
+
+
+def test_layer_c3_skewed_scale(hip, oracle):
+    """DeepSeek-V3-scale layer with a Zipf(1.1) correction bias: about 10 % of the experts take about half of the
+    assignments; stresses the three-phase permutation and experts with thousands of rows."""
+    cfg = synth.CONFIGS["c3"]
+    v = _scale_check(hip, oracle, cfg, n_sample=6)
+    counts = np.sort(v["counts"])[::-1]
+    top = counts[: cfg.n_experts // 10].sum() / counts.sum()
+    assert 0.35 <= top <= 0.65, top
