@@ -6,6 +6,16 @@
 
 namespace fe {
 
+// Activation scales are kept in the order the MFMA scale operand wants them: the e8m0 byte of the 32-wide k
+// block b (k step kt = b/4, quarter g = b%4) sits at byte scale_pos(b) of its row, so that lane (column, g)
+// reads the four k steps kt4*4 .. kt4*4+3 of its quarter as one dword at 16*kt4 + 4*g and selects the step
+// with op_sel.  Rows are scale_pitch(K) bytes long.
+__host__ __device__ __forceinline__ int scale_pos(int b) {
+    const int kt = b >> 2, g = b & 3;
+    return (kt >> 2) * 16 + g * 4 + (kt & 3);
+}
+__host__ __device__ __forceinline__ int scale_pitch(int K) { return ((K / 128 + 3) / 4) * 16; }
+
 // act_quant_fp8 of one block of 32 consecutive values (crates/ferrite-models/src/dsv41/quant.rs:190-214,
 // power-of-two scale): 32 e4m3 codes to q (32-byte aligned) and the e8m0 scale byte as the return value.
 template <typename XT>

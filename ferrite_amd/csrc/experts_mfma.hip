@@ -13,6 +13,7 @@
 // code tiles in exactly the order a wave consumes them: [item][k step][tile 0..3][lane][16 B], so a wave
 // reads one contiguous 4 KiB per k step with 128-bit loads; scales are [item][4 k steps][lane][tile][4 B].
 #include "internal.hpp"
+#include "device_utils.hpp"
 #include "numerics.hpp"
 
 namespace fe {
@@ -161,7 +162,8 @@ __device__ __forceinline__ void stream_item(StreamRegs& r, const u4v* __restrict
 }
 
 // Copies the e4m3 rows of a unit into LDS in B-operand order and builds the packed scale words.
-// row_src(c) gives the source row index of column c (or -1).  q rows are K bytes, scale rows K/32 bytes.
+// row_src(c) gives the source row index of column c (or -1).  q rows are K bytes; scale rows are in operand
+// order (scale_pos), scale_pitch(K) bytes long.
 template <typename RowFn>
 __device__ __forceinline__ void fill_b_operand(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs, int K,
                                                int nrows, RowFn row_src, u4v* bq, uint32_t* bsc) {
@@ -181,14 +183,7 @@ __device__ __forceinline__ void fill_b_operand(const uint8_t* __restrict__ q, co
         uint32_t v = 0x7f7f7f7fu;
         if (c < nrows) {
             const int r = row_src(c);
-            if (r >= 0) {
-                v = 0;
-                for (int qq = 0; qq < 4; ++qq) {
-                    int kt = k4 * 4 + qq;
-                    uint32_t b = kt < KT ? qs[(size_t)r * (K / 32) + kt * 4 + g] : 127u;
-                    v |= b << (8 * qq);
-                }
-            }
+            if (r >= 0) v = *reinterpret_cast<const uint32_t*>(qs + (size_t)r * scale_pitch(K) + k4 * 16 + g * 4);
         }
         bsc[idx] = v;
     }
@@ -201,14 +196,14 @@ struct MfmaArgs {
     const uint8_t* sh_scales;
     size_t codes_per_expert, scales_per_expert;
     const int32_t *unit_expert, *unit_row0, *unit_rows, *n_units;
-    int n, topk, n_experts, hidden, inter, shared_inter, act_ld;
+    int n, topk, n_experts, hidden, inter, shared_inter, act_ld, unit_cap;
     float limit;
 };
 
 // A unit read from device tables is used only if it is well formed.
 __device__ __forceinline__ bool unit_ok(const MfmaArgs& a, int e, int row0, int nrows) {
     const int nk = a.n * a.topk;
-    if (nrows < 1 || nrows > 16 || row0 < 0) return false;
+    if (nrows < 1 || nrows > a.unit_cap || row0 < 0) return false;
     if (e == a.n_experts) return a.shared_inter > 0 && row0 >= nk && row0 + nrows <= nk + a.n;
     return e >= 0 && e < a.n_experts && row0 + nrows <= nk;
 }
@@ -281,7 +276,7 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
         uint8_t* dst = act_q + (size_t)(row0 + c) * a.act_ld + (size_t)item * 32 + g * 4;
         *reinterpret_cast<uint32_t*>(dst) = p0;
         *reinterpret_cast<uint32_t*>(dst + 16) = p1;
-        if (g == 0) act_s[(size_t)(row0 + c) * (a.act_ld / 32) + item] = (uint8_t)sb;
+        if (g == 0) act_s[(size_t)(row0 + c) * scale_pitch(a.act_ld) + scale_pos(item)] = (uint8_t)sb;
     }
 }
 
@@ -322,14 +317,8 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
         for (int idx = threadIdx.x; idx < KT4 * 64; idx += blockDim.x) {
             const int k4 = idx >> 6, l = idx & 63, c = l & 15, g = l >> 4;
             uint32_t v = 0x7f7f7f7fu;
-            if (c < nrows) {
-                v = 0;
-                for (int qq = 0; qq < 4; ++qq) {
-                    int kt = k4 * 4 + qq;
-                    uint32_t b = kt < KT ? act_s[(size_t)(row0 + c) * (a.act_ld / 32) + kt * 4 + g] : 127u;
-                    v |= b << (8 * qq);
-                }
-            }
+            if (c < nrows)
+                v = *reinterpret_cast<const uint32_t*>(act_s + (size_t)(row0 + c) * scale_pitch(a.act_ld) + k4 * 16 + g * 4);
             bsc[idx] = v;
         }
     }
@@ -357,6 +346,278 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
     }
 }
 
+
+// ---- prefill kernels: units of up to 128 rows ------------------------------------------------------------
+// One block (4 waves) computes 4 items (128 gate + 128 up rows, or 256 down rows) x 128 grouped rows of one unit.
+// Both operands go through LDS, one k step (128 k) per stage, two stages; the loads of k step kt+2 are issued
+// into registers before the MFMAs of k step kt and reach LDS after those of kt+1.  Wave w owns items
+// 2*(w&1), 2*(w&1)+1 and rows 64*(w>>1) .. +63: 8 weight tiles x 4 row tiles = 32 MFMAs per k step.
+// Accumulation order over k is the same as in the 16-row kernels, so both give the same bits.
+constexpr int PF_ROWS = 128;
+constexpr int PF_ITEMS = 4;
+constexpr int PF_LDS_STAGE = 2 * 1024;                 // u4v per stage: 1024 weight slots + 1024 activation slots
+constexpr size_t PF_LDS_BYTES = 2 * PF_LDS_STAGE * 16;  // 64 KiB
+
+struct PfStage {
+    u4v a[4], b[4];
+};
+
+struct PfSrc {
+    const u4v* a[4];       // this thread's slot of k step 0 of each staged item
+    const uint8_t* b[4];   // this thread's 16 bytes of k step 0 of each staged row
+};
+
+__device__ __forceinline__ void pf_load(PfStage& s, const PfSrc& p, int kt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s.a[i] = p.a[i][(size_t)kt * 256];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s.b[i] = *reinterpret_cast<const u4v*>(p.b[i] + (size_t)kt * 128);
+}
+
+// Activation slots are XOR-swizzled: row c of a 16-row tile, 16-byte chunk j = 4*half + g of the k step sits
+// at slot half*64 + g*16 + (c ^ j), so the 8 chunks of a row (written by 8 neighbouring lanes) fall into
+// different banks while a 16-lane operand read still covers 16 consecutive slots.
+__device__ __forceinline__ void pf_store(const PfStage& s, u4v* stage, int t, int bslot) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stage[i * 256 + t] = s.a[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stage[1024 + bslot + i * 256] = s.b[i];
+}
+
+template <int Q>
+__device__ __forceinline__ void pf_compute(const u4v* stage, int wi, int wt, int lane, const u4v (&asc)[2],
+                                           const uint32_t (&bsc)[4], v4f (&acc)[2][4][4]) {
+    const int g = lane >> 4, cc = lane & 15;
+    v8i bv[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+        const u4v* bt = stage + 1024 + (wt * 4 + tt) * 128;
+        const u4v b0 = bt[g * 16 + (cc ^ g)];
+        const u4v b1 = bt[64 + g * 16 + (cc ^ (4 + g))];
+        bv[tt] = (v8i){(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+    }
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+        const uint32_t scs[4] = {asc[ii][0], asc[ii][1], asc[ii][2], asc[ii][3]};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const u4v av = stage[((wi * 2 + ii) * 4 + t) * 64 + lane];
+            const v8i a8 = {(int)av[0], (int)av[1], (int)av[2], (int)av[3], 0, 0, 0, 0};
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+                acc[ii][t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    a8, bv[tt], acc[ii][t][tt], 4 /*A e2m1*/, 0 /*B e4m3*/, Q, (int)scs[t], Q, (int)bsc[tt]);
+        }
+    }
+}
+
+struct PfCtx {
+    PfSrc src;
+    const u4v* asp[2];        // weight scale words of the wave's two items
+    const uint8_t* bsp[4];    // activation scale rows of the lane's column in the wave's 4 row tiles
+    int KT, t, bslot, wi, wt, lane;
+};
+
+template <int Q>
+__device__ __forceinline__ void pf_step(const PfCtx& c, PfStage (&st)[2], u4v* lds, int kt, const u4v (&asc)[2],
+                                        const uint32_t (&bsc)[4], v4f (&acc)[2][4][4]) {
+    if (kt >= c.KT) return;
+    if (kt + 2 < c.KT) pf_load(st[Q & 1], c.src, kt + 2);
+    pf_compute<Q>(lds + (Q & 1) * PF_LDS_STAGE, c.wi, c.wt, c.lane, asc, bsc, acc);
+    if (kt + 1 < c.KT) pf_store(st[(Q + 1) & 1], lds + ((Q + 1) & 1) * PF_LDS_STAGE, c.t, c.bslot);
+    __syncthreads();
+}
+
+__device__ __forceinline__ void pf_mainloop(const PfCtx& c, u4v* lds, v4f (&acc)[2][4][4]) {
+    const int KT4 = (c.KT + 3) >> 2, g = c.lane >> 4;
+    PfStage st[2];
+    pf_load(st[0], c.src, 0);
+    if (c.KT > 1) pf_load(st[1], c.src, 1);
+    u4v asc[2], asc_n[2];
+    uint32_t bsc[4], bsc_n[4];
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) asc[ii] = asc_n[ii] = c.asp[ii][c.lane];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) bsc[tt] = bsc_n[tt] = *reinterpret_cast<const uint32_t*>(c.bsp[tt] + g * 4);
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) acc[ii][t][tt] = (v4f){0.f, 0.f, 0.f, 0.f};
+    pf_store(st[0], lds, c.t, c.bslot);
+    __syncthreads();
+#pragma unroll 1
+    for (int g4 = 0; g4 < KT4; ++g4) {
+        if (g4 + 1 < KT4) {
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii) asc_n[ii] = c.asp[ii][(size_t)(g4 + 1) * 64 + c.lane];
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+                bsc_n[tt] = *reinterpret_cast<const uint32_t*>(c.bsp[tt] + (g4 + 1) * 16 + g * 4);
+        }
+        const int kt = g4 * 4;
+        pf_step<0>(c, st, lds, kt, asc, bsc, acc);
+        pf_step<1>(c, st, lds, kt + 1, asc, bsc, acc);
+        pf_step<2>(c, st, lds, kt + 2, asc, bsc, acc);
+        pf_step<3>(c, st, lds, kt + 3, asc, bsc, acc);
+#pragma unroll
+        for (int ii = 0; ii < 2; ++ii) asc[ii] = asc_n[ii];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) bsc[tt] = bsc_n[tt];
+    }
+}
+
+// Block -> (unit, item group).  Hardware deals consecutive blocks round-robin over the 8 XCDs; the live work
+// (n_units * groups) is cut into 8 contiguous ranges, one per XCD, so that the blocks of one unit, and mostly
+// of one expert, share an L2.  Returns false for blocks without work.
+__device__ __forceinline__ bool pf_block_work(int n_units, int groups, int& u, int& ig) {
+    const int total = n_units * groups, per_xcd = (total + 7) >> 3;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int v = xcd * per_xcd + slot;
+    if (slot >= per_xcd || v >= total) return false;
+    u = v / groups;
+    ig = v - u * groups;
+    return true;
+}
+
+// Fills the block-level part of the context.  row_q(c) returns the e4m3 row of unit column c, row_s(c) its
+// scale row; columns >= nrows alias column 0 (their results are never stored).
+template <typename RowQ, typename RowS>
+__device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const uint8_t* sbase, int item0, int items,
+                                           int KT, int nrows, RowQ row_q, RowS row_s) {
+    const int t = threadIdx.x, KT4 = (KT + 3) >> 2;
+    c.KT = KT; c.t = t; c.lane = t & 63;
+    const int wave = t >> 6;
+    c.wi = wave & 1; c.wt = wave >> 1;
+    const int j = t & 7, r8 = t >> 3;   // chunk of the k step, row within a group of 32 rows
+    c.bslot = (r8 >> 4) * 128 + (j >> 2) * 64 + (j & 3) * 16 + ((r8 & 15) ^ j);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int item = min(item0 + i, items - 1);
+        c.src.a[i] = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256 + t;
+        const int col = r8 + 32 * i;
+        c.src.b[i] = row_q(col < nrows ? col : 0) + j * 16;
+    }
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+        const int item = min(item0 + c.wi * 2 + ii, items - 1);
+        c.asp[ii] = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
+    }
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+        const int col = (c.wt * 4 + tt) * 16 + (c.lane & 15);
+        c.bsp[tt] = row_s(col < nrows ? col : 0);
+    }
+}
+
+__global__ __launch_bounds__(256) void gate_up_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
+                                                              const uint8_t* __restrict__ xs,
+                                                              const int32_t* __restrict__ gather_src,
+                                                              uint8_t* __restrict__ act_q,
+                                                              uint8_t* __restrict__ act_s) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int u, ig;
+    if (!pf_block_work(*a.n_units, groups, u, ig)) return;
+    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    if (!unit_ok(a, e, row0, nrows)) return;
+    const bool shared = e == a.n_experts;
+    const int inter = shared ? a.shared_inter : a.inter;
+    const int items = inter / 32, item0 = ig * PF_ITEMS;
+    if (item0 >= items) return;
+    const int H = a.hidden, nk = a.n * a.topk, topk = a.topk, n = a.n;
+    const int spitch = scale_pitch(H);
+    auto token = [&](int col) -> int {
+        const int gr = row0 + col;
+        if (shared) return gr - nk;
+        const int i = gather_src[gr];
+        const int tk = (i < 0 || i >= nk) ? 0 : i / topk;
+        return tk < n ? tk : 0;
+    };
+    PfCtx c;
+    pf_context(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
+               shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, item0, items, H / 128, nrows,
+               [&](int col) { return xq + (size_t)token(col) * H; },
+               [&](int col) { return xs + (size_t)token(col) * spitch; });
+    v4f acc[2][4][4];
+    pf_mainloop(c, reinterpret_cast<u4v*>(lds_raw), acc);
+
+    const int cc = c.lane & 15, g = c.lane >> 4;
+    const int apitch = scale_pitch(a.act_ld);
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+        const int item = item0 + c.wi * 2 + ii;
+        if (item >= items) break;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            const int col = (c.wt * 4 + tt) * 16 + cc;
+            float r0[4], r1[4];
+            float amax = 0.0f;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                r0[v] = swiglu_ref(acc[ii][0][tt][v], acc[ii][2][tt][v], a.limit);
+                r1[v] = swiglu_ref(acc[ii][1][tt][v], acc[ii][3][tt][v], a.limit);
+                amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+            }
+            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            if (col < nrows) {
+                const uint32_t sb = block_scale_e8m0(amax);
+                const float inv = u2f((254u - sb) << 23);
+                uint32_t p0 = 0, p1 = 0;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    p0 |= e4m3_encode(r0[v] * inv) << (8 * v);
+                    p1 |= e4m3_encode(r1[v] * inv) << (8 * v);
+                }
+                uint8_t* dst = act_q + (size_t)(row0 + col) * a.act_ld + (size_t)item * 32 + g * 4;
+                *reinterpret_cast<uint32_t*>(dst) = p0;
+                *reinterpret_cast<uint32_t*>(dst + 16) = p1;
+                if (g == 0) act_s[(size_t)(row0 + col) * apitch + scale_pos(item)] = (uint8_t)sb;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void down_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
+                                                           const uint8_t* __restrict__ act_s, float* __restrict__ y) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int u, ig;
+    if (!pf_block_work(*a.n_units, groups, u, ig)) return;
+    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    if (!unit_ok(a, e, row0, nrows)) return;
+    const bool shared = e == a.n_experts;
+    const int inter = shared ? a.shared_inter : a.inter;
+    const int H = a.hidden, items = H / 64, item0 = ig * PF_ITEMS;
+    if (item0 >= items) return;
+    const int apitch = scale_pitch(a.act_ld), act_ld = a.act_ld;
+    PfCtx c;
+    pf_context(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
+               shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, item0, items, inter / 128, nrows,
+               [&](int col) { return act_q + (size_t)(row0 + col) * act_ld; },
+               [&](int col) { return act_s + (size_t)(row0 + col) * apitch; });
+    v4f acc[2][4][4];
+    pf_mainloop(c, reinterpret_cast<u4v*>(lds_raw), acc);
+
+    const int cc = c.lane & 15, g = c.lane >> 4;
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+        const int item = item0 + c.wi * 2 + ii;
+        if (item >= items) break;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            const int col = (c.wt * 4 + tt) * 16 + cc;
+            if (col < nrows) {
+                float* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    *reinterpret_cast<float4*>(dst + t * 16) =
+                        make_float4(acc[ii][t][tt][0], acc[ii][t][tt][1], acc[ii][t][tt][2], acc[ii][t][tt][3]);
+            }
+        }
+    }
+}
+
 // ---- launchers ----------------------------------------------------------------------------------------
 constexpr int GU_WAVES = 4;
 constexpr int DN_WAVES = 4;
@@ -377,6 +638,7 @@ static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int
     a.shared_inter = s.shared_inter;
     a.act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
     a.limit = s.swiglu_limit;
+    a.unit_cap = units.unit_rows_cap;
     return a;
 }
 
@@ -396,9 +658,18 @@ static int set_lds_limit(K kernel, size_t bytes, size_t* raised) {
 int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
                         int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
                         hipStream_t st) {
-    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
     MfmaArgs a = make_args(s, packed, n, units, false);
     const int imax = a.act_ld;
+    if (units.unit_rows_cap == PF_ROWS) {
+        static size_t raised_pf = 0;
+        int rc = set_lds_limit(gate_up_prefill_kernel, PF_LDS_BYTES, &raised_pf);
+        if (rc) return rc;
+        const int groups = (imax / 32 + PF_ITEMS - 1) / PF_ITEMS;
+        const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+        gate_up_prefill_kernel<<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, xq, xs, gather_src, act_q, act_s);
+        return check_launch("gate_up_prefill");
+    }
+    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = (size_t)s.hidden * 16 + (size_t)((s.hidden / 128 + 3) / 4) * 256;
     static size_t raised = 0;
     int rc = set_lds_limit(gate_up_mfma_kernel<GU_WAVES>, lds, &raised);
@@ -410,8 +681,17 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
 
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
                      int n, const UnitTables& units, float* y, hipStream_t st) {
-    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
     MfmaArgs a = make_args(s, packed, n, units, true);
+    if (units.unit_rows_cap == PF_ROWS) {
+        static size_t raised_pf = 0;
+        int rc = set_lds_limit(down_prefill_kernel, PF_LDS_BYTES, &raised_pf);
+        if (rc) return rc;
+        const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
+        const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+        down_prefill_kernel<<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, y);
+        return check_launch("down_prefill");
+    }
+    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = (size_t)a.act_ld * 16 + (size_t)((a.act_ld / 128 + 3) / 4) * 256;
     static size_t raised = 0;
     int rc = set_lds_limit(down_mfma_kernel<DN_WAVES, DN_IPW>, lds, &raised);

@@ -32,23 +32,28 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t* __res
 }
 
 // One thread quantises one block of 32 consecutive values of a row.
+// operand_order: scales go to scale_pos() within rows of scale_pitch(cols) bytes instead of row-major.
 template <typename XT>
-__global__ __launch_bounds__(256) void act_quant_kernel(const XT* __restrict__ x, int64_t nblocks,
-                                                        uint8_t* __restrict__ q, uint8_t* __restrict__ scale) {
+__global__ __launch_bounds__(256) void act_quant_kernel(const XT* __restrict__ x, int64_t nblocks, int bpr,
+                                                        int operand_order, uint8_t* __restrict__ q,
+                                                        uint8_t* __restrict__ scale) {
     int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nblocks) return;
-    scale[b] = (uint8_t)quant_block32(x + b * 32, q + b * 32);
+    const uint8_t sb = (uint8_t)quant_block32(x + b * 32, q + b * 32);
+    if (operand_order) scale[(b / bpr) * scale_pitch(bpr * 32) + scale_pos((int)(b % bpr))] = sb;
+    else scale[b] = sb;
 }
 
-int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, hipStream_t st) {
+int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, int operand_order,
+                     hipStream_t st) {
     if (rows < 0 || cols < 0 || cols % 32 != 0) return FERRITE_ERR_INVALID_ARG;
     int64_t nblocks = rows * (cols / 32);
     if (nblocks == 0) return FERRITE_OK;
     unsigned grid = (unsigned)((nblocks + 255) / 256);
     if (x_dtype == FERRITE_DT_F32)
-        act_quant_kernel<float><<<grid, 256, 0, st>>>((const float*)x, nblocks, q, scale);
+        act_quant_kernel<float><<<grid, 256, 0, st>>>((const float*)x, nblocks, cols / 32, operand_order, q, scale);
     else if (x_dtype == FERRITE_DT_BF16)
-        act_quant_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)x, nblocks, q, scale);
+        act_quant_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)x, nblocks, cols / 32, operand_order, q, scale);
     else
         return FERRITE_ERR_INVALID_ARG;
     return check_launch("act_quant");
@@ -73,5 +78,5 @@ extern "C" int ferrite_act_quant_fp8(const void* x, int x_dtype, int64_t rows, i
                                      ferrite_stream_t stream) {
     if (rows > 0 && cols > 0 && (!x || !q || !scale)) return FERRITE_ERR_INVALID_ARG;
     if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(q) & 15)) return FERRITE_DECLINED;
-    return launch_act_quant(x, x_dtype, rows, cols, q, scale, as_stream(stream));
+    return launch_act_quant(x, x_dtype, rows, cols, q, scale, 0, as_stream(stream));
 }

@@ -33,6 +33,11 @@ inline int max_units_for(int n, int topk, int n_experts, int has_shared, int uni
     return (int)u;
 }
 
+// Rows per unit for a layer call: 128-row units (both GEMM operands tiled through LDS) once the average expert
+// sees enough rows to fill them, 16-row units (weights streamed once per unit) below that.  The environment
+// variable FERRITE_HIP_UNIT_ROWS (16 or 128) overrides the choice; it is read at every call.
+int unit_rows_for(int n, int topk, int n_experts);
+
 // route.hip
 int launch_matmul_exact(const void* x, int x_dtype, const float* w, const float* bias, float* out, int n, int k,
                         int o, hipStream_t st);
@@ -75,6 +80,7 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ui
                      int n, const UnitTables& units, float* y, hipStream_t st);
 
 // formats.hip
-int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, hipStream_t st);
+int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, int operand_order,
+                     hipStream_t st);
 
 }  // namespace fe

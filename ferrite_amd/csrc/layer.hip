@@ -2,6 +2,7 @@
 // The driver only enqueues kernels on the caller's stream: no allocation, no synchronisation, no host reads
 // of device data, and a launch sequence that is a function of (shape, n, mode) alone.
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "internal.hpp"
@@ -31,8 +32,16 @@ struct Workspace {
     size_t unit_expert, unit_row0, unit_rows, n_units, perm_scratch, perm_scratch_bytes, counters;
     size_t xq, xs, act, act_s, y;
     size_t total;
-    int max_units, rows;
+    int max_units, rows, unit_cap;
 };
+
+int unit_rows_for(int n, int topk, int n_experts) {
+    if (const char* v = getenv("FERRITE_HIP_UNIT_ROWS")) {
+        if (!strcmp(v, "16")) return 16;
+        if (!strcmp(v, "128")) return 128;
+    }
+    return (long)n * topk >= 48L * n_experts ? 128 : 16;
+}
 
 static size_t bump(size_t& off, size_t bytes) {
     size_t at = off;
@@ -46,7 +55,8 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     const int has_shared = s.shared_inter > 0;
     const size_t act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
     w.rows = (int)(nk + (has_shared ? n : 0));
-    w.max_units = max_units_for(n, s.topk, s.n_experts, has_shared, 16);
+    w.unit_cap = mode == FERRITE_MODE_MFMA_FP8 ? unit_rows_for(n, s.topk, s.n_experts) : 16;
+    w.max_units = max_units_for(n, s.topk, s.n_experts, has_shared, w.unit_cap);
     size_t off = 0;
     w.counters = bump(off, ((size_t)n + 1) * 4);   // first: ferrite_moe_layer_workspace_init clears it
     w.logits = bump(off, (size_t)n * E * 4);
@@ -67,9 +77,9 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     w.perm_scratch = bump(off, w.perm_scratch_bytes);
     if (mode == FERRITE_MODE_MFMA_FP8) {
         w.xq = bump(off, (size_t)n * H);
-        w.xs = bump(off, (size_t)n * (H / 32));
+        w.xs = bump(off, (size_t)n * (((H / 128 + 3) / 4) * 16));
         w.act = bump(off, (size_t)w.rows * act_ld);
-        w.act_s = bump(off, (size_t)w.rows * (act_ld / 32));
+        w.act_s = bump(off, (size_t)w.rows * (((act_ld / 128 + 3) / 4) * 16));
     } else {
         w.act = bump(off, (size_t)w.rows * act_ld * 4);
     }
@@ -179,7 +189,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     float* y = reinterpret_cast<float*>(b + w.y);
 
     UnitTables units{reinterpret_cast<int32_t*>(b + w.unit_expert), reinterpret_cast<int32_t*>(b + w.unit_row0),
-                     reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.n_units), 16,
+                     reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.n_units), w.unit_cap,
                      w.max_units};
     uint8_t* xq = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xq) : nullptr;
     uint8_t* xs = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xs) : nullptr;
@@ -222,7 +232,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         return rc;
     if ((rc = mark(ev, 3, st))) return rc;
     if (xq) {
-        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq, xs, st))) return rc;
+        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq, xs, 1, st))) return rc;
     }
     if ((rc = mark(ev, 4, st))) return rc;
     }

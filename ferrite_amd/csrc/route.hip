@@ -569,7 +569,8 @@ __global__ __launch_bounds__(64) void moe_head_kernel(HeadArgs a) {
     const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
     if (eb == eblocks) {
         for (int b = lane; b < H / 32; b += 64)
-            a.xs[(size_t)t * (H / 32) + b] = (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
+            a.xs[(size_t)t * scale_pitch(H) + scale_pos(b)] =
+                (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
         return;
     }
     float4* xl = reinterpret_cast<float4*>(head_lds);

@@ -91,6 +91,25 @@ def test_layer_small_shapes_both_modes(hip, oracle, seed, n):
     assert max_abs_rel(out, oracle.moe_ffn_mxfp4(inp, act_mode=1)["out"]) <= TOL_MFMA
 
 
+@pytest.mark.parametrize("seed,n,hidden,inter,shared", [(5, 8, 256, 128, 128), (6, 150, 256, 256, 128),
+                                                        (7, 700, 384, 256, 384), (8, 1100, 512, 128, 0)])
+def test_unit_rows_128_equals_16(hip, oracle, monkeypatch, seed, n, hidden, inter, shared):
+    """The 128-row-unit kernels (both operands tiled through LDS) accumulate over k in the same order as the 16-row
+    ones: identical bits, on ragged units (1..128 rows, several units per expert, H/64 not a multiple of the block's
+    4 items), and the result is within the MFMA bar of the oracle."""
+    cfg = synth.MoeConfig(n, hidden, 8, 3, inter, shared, 4, 2)
+    inp = synth.make_inputs(cfg, seed=seed)
+    layer = hip.load_moe_layer(inp)
+    outs = {}
+    for rows in ("16", "128"):
+        monkeypatch.setenv("FERRITE_HIP_UNIT_ROWS", rows)
+        layer._ws.clear()
+        outs[rows], v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    layer._ws.clear()
+    assert np.array_equal(outs["16"], outs["128"])
+    assert max_abs_rel(outs["128"], oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
+
+
 def test_layer_c1_decode(hip, oracle):
     """The decode benchmark shape: 32 tokens, H 4096, 128 experts, top-8 of 8 groups, I 1536, bf16 activations."""
     inp = synth.make_inputs(synth.CONFIGS["c1"], seed=0)
