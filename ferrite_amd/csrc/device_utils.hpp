@@ -16,6 +16,30 @@ __host__ __device__ __forceinline__ int scale_pos(int b) {
 }
 __host__ __device__ __forceinline__ int scale_pitch(int K) { return ((K / 128 + 3) / 4) * 16; }
 
+// Four floats to four packed e4m3 codes (byte i = value i) with the hardware converter (round to nearest even),
+// made to agree with e4m3_encode(): magnitudes are clamped to 448 first, and the reference's subnormal rule
+// (quant.rs:98-124: |x| in [7.5, 8) * 2^-9 encodes as 7, not as the smallest normal) is applied by moving such
+// values onto 7 * 2^-9 before the conversion.  Anything that is not <= 448 in magnitude, NaN included, becomes
+// +-448 as in e4m3_encode().
+__device__ __forceinline__ float e4m3_prepare(float x) {
+    const float ax = fabsf(x);
+    x = (ax >= 0x1.ep-7f && ax < 0x1p-6f) ? copysignf(0x1.cp-7f, x) : x;
+    return ax <= 448.0f ? x : copysignf(448.0f, x);
+}
+__device__ __forceinline__ uint32_t e4m3_encode4_hw(float a, float b, float c, float d) {
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(e4m3_prepare(a), e4m3_prepare(b), 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(e4m3_prepare(c), e4m3_prepare(d), w, true);
+    return (uint32_t)w;
+}
+
+// Clamped SwiGLU (cpu.rs:192-201) for the MFMA mode, whose results are rounded to e4m3 right afterwards: the
+// hardware exponential and reciprocal (a few ulp) instead of the bit-exact expf and division of swiglu_ref().
+__device__ __forceinline__ float swiglu_fast(float g, float u, float limit) {
+    const float gi = fminf(g, limit);
+    const float ui = fminf(fmaxf(u, -limit), limit);
+    return gi * __builtin_amdgcn_rcpf(1.0f + __expf(-gi)) * ui;
+}
+
 // act_quant_fp8 of one block of 32 consecutive values (crates/ferrite-models/src/dsv41/quant.rs:190-214,
 // power-of-two scale): 32 e4m3 codes to q (32-byte aligned) and the e8m0 scale byte as the return value.
 template <typename XT>
@@ -49,8 +73,7 @@ __device__ __forceinline__ uint32_t quant_block32(const XT* __restrict__ src, ui
     uint32_t out[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        out[i] = e4m3_encode(v[4 * i] * inv) | (e4m3_encode(v[4 * i + 1] * inv) << 8) |
-                 (e4m3_encode(v[4 * i + 2] * inv) << 16) | (e4m3_encode(v[4 * i + 3] * inv) << 24);
+        out[i] = e4m3_encode4_hw(v[4 * i] * inv, v[4 * i + 1] * inv, v[4 * i + 2] * inv, v[4 * i + 3] * inv);
     }
     uint4* o = reinterpret_cast<uint4*>(q);
     o[0] = make_uint4(out[0], out[1], out[2], out[3]);

@@ -257,8 +257,8 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
     float amax = 0.0f;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-        r0[v] = swiglu_ref(acc[0][v], acc[2][v], a.limit);
-        r1[v] = swiglu_ref(acc[1][v], acc[3][v], a.limit);
+        r0[v] = swiglu_fast(acc[0][v], acc[2][v], a.limit);
+        r1[v] = swiglu_fast(acc[1][v], acc[3][v], a.limit);
         amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
     }
     amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
@@ -267,12 +267,8 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
     if (c < nrows) {
         const uint32_t sb = block_scale_e8m0(amax);
         const float inv = u2f((254u - sb) << 23);
-        uint32_t p0 = 0, p1 = 0;
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            p0 |= e4m3_encode(r0[v] * inv) << (8 * v);
-            p1 |= e4m3_encode(r1[v] * inv) << (8 * v);
-        }
+        const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
+        const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
         uint8_t* dst = act_q + (size_t)(row0 + c) * a.act_ld + (size_t)item * 32 + g * 4;
         *reinterpret_cast<uint32_t*>(dst) = p0;
         *reinterpret_cast<uint32_t*>(dst + 16) = p1;
@@ -349,123 +345,130 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
 
 // ---- prefill kernels: units of up to 128 rows ------------------------------------------------------------
 // One block (4 waves) computes 4 items (128 gate + 128 up rows, or 256 down rows) x 128 grouped rows of one unit.
-// Both operands go through LDS, one k step (128 k) per stage, two stages; the loads of k step kt+2 are issued
-// into registers before the MFMAs of k step kt and reach LDS after those of kt+1.  Wave w owns items
-// 2*(w&1), 2*(w&1)+1 and rows 64*(w>>1) .. +63: 8 weight tiles x 4 row tiles = 32 MFMAs per k step.
+// Both operands go through LDS, one k step (128 k) per stage, two stages, filled by direct global->LDS loads
+// (global_load_lds_dwordx4: lane l of the issuing wave lands at base + 16*l, so the lane -> source address map
+// alone produces the operand order; no staging registers, no LDS write instructions).  Wave w fills item w and
+// row tiles 2w, 2w+1 of the next stage while the MFMAs of the current one run; it computes items 2*(w&1),
+// 2*(w&1)+1 x rows 64*(w>>1) .. +63: 8 weight tiles x 4 row tiles = 32 MFMAs per k step.  128 accumulator
+// registers + <= 128 others let two blocks share a CU, so one block's stage hand-over (wait for the loads,
+// barrier, operand reads) hides behind the other's MFMAs.
 // Accumulation order over k is the same as in the 16-row kernels, so both give the same bits.
 constexpr int PF_ROWS = 128;
 constexpr int PF_ITEMS = 4;
 constexpr int PF_LDS_STAGE = 2 * 1024;                 // u4v per stage: 1024 weight slots + 1024 activation slots
 constexpr size_t PF_LDS_BYTES = 2 * PF_LDS_STAGE * 16;  // 64 KiB
 
-struct PfStage {
-    u4v a[4], b[4];
-};
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void glb_void;
 
-struct PfSrc {
-    const u4v* a[4];       // this thread's slot of k step 0 of each staged item
-    const uint8_t* b[4];   // this thread's 16 bytes of k step 0 of each staged row
-};
-
-__device__ __forceinline__ void pf_load(PfStage& s, const PfSrc& p, int kt) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s.a[i] = p.a[i][(size_t)kt * 256];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) s.b[i] = *reinterpret_cast<const u4v*>(p.b[i] + (size_t)kt * 128);
+// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane (lds_base wave-uniform).
+__device__ __forceinline__ void dma16(const void* g, void* lds_base) {
+    __builtin_amdgcn_global_load_lds((glb_void*)g, (lds_void*)lds_base, 16, 0, 0);
 }
 
-// Activation slots are XOR-swizzled: row c of a 16-row tile, 16-byte chunk j = 4*half + g of the k step sits
-// at slot half*64 + g*16 + (c ^ j), so the 8 chunks of a row (written by 8 neighbouring lanes) fall into
-// different banks while a 16-lane operand read still covers 16 consecutive slots.
-__device__ __forceinline__ void pf_store(const PfStage& s, u4v* stage, int t, int bslot) {
+struct PfCtx {
+    const u4v* a_src;         // codes of the item this wave stages, k step 0, + lane
+    const uint8_t* b_src[2];  // e4m3 rows (2*wave+i)*16 + lane%16 of the unit, + 16*(lane/16)
+    const u4v* asp[2];        // weight scale words of the wave's two items
+    const uint8_t* bsp[4];    // activation scale rows of the lane's column in the wave's 4 row tiles
+    int KT, wave, wi, wt, lane;
+};
+
+// Starts the loads of k step kt into `stage`.
+__device__ __forceinline__ void pf_fill(const PfCtx& c, u4v* stage, int kt) {
+    const u4v* a = c.a_src + (size_t)kt * 256;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) stage[i * 256 + t] = s.a[i];
+    for (int t = 0; t < 4; ++t) dma16(a + t * 64, stage + (c.wave * 4 + t) * 64);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) stage[1024 + bslot + i * 256] = s.b[i];
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            dma16(c.b_src[i] + (size_t)kt * 128 + h * 64, stage + 1024 + ((c.wave * 2 + i) * 2 + h) * 64);
 }
 
+// All loads into LDS issued by this wave have landed (vmcnt 0; expcnt and lgkmcnt left alone).
+__device__ __forceinline__ void pf_wait_fill() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// One k step: operands of the current stage into registers, then the next stage's loads are started (after the
+// operand reads in program order: the compiler cannot tell the two stages apart and would otherwise wait for the
+// loads before it reads), then the MFMAs; the step ends when the next stage is complete for every wave.
 template <int Q>
-__device__ __forceinline__ void pf_compute(const u4v* stage, int wi, int wt, int lane, const u4v (&asc)[2],
-                                           const uint32_t (&bsc)[4], v4f (&acc)[2][4][4]) {
-    const int g = lane >> 4, cc = lane & 15;
+__device__ __forceinline__ void pf_step(const PfCtx& c, u4v* lds, int kt, const u4v (&asc)[2],
+                                        const uint32_t (&bsc)[4], v4f (&acc)[2][4][4]) {
+    const u4v* cur = lds + (Q & 1) * PF_LDS_STAGE;
     v8i bv[4];
+    u4v av[2][4];
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
-        const u4v* bt = stage + 1024 + (wt * 4 + tt) * 128;
-        const u4v b0 = bt[g * 16 + (cc ^ g)];
-        const u4v b1 = bt[64 + g * 16 + (cc ^ (4 + g))];
+        const u4v* bt = cur + 1024 + (c.wt * 4 + tt) * 128;
+        const u4v b0 = bt[c.lane];
+        const u4v b1 = bt[64 + c.lane];
         bv[tt] = (v8i){(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
     }
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) av[ii][t] = cur[((c.wi * 2 + ii) * 4 + t) * 64 + c.lane];
+    __builtin_amdgcn_sched_barrier(0);
+    pf_fill(c, lds + ((Q + 1) & 1) * PF_LDS_STAGE, min(kt + 1, c.KT - 1));
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
         const uint32_t scs[4] = {asc[ii][0], asc[ii][1], asc[ii][2], asc[ii][3]};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const u4v av = stage[((wi * 2 + ii) * 4 + t) * 64 + lane];
-            const v8i a8 = {(int)av[0], (int)av[1], (int)av[2], (int)av[3], 0, 0, 0, 0};
+            const v8i a8 = {(int)av[ii][t][0], (int)av[ii][t][1], (int)av[ii][t][2], (int)av[ii][t][3], 0, 0, 0, 0};
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt)
                 acc[ii][t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                     a8, bv[tt], acc[ii][t][tt], 4 /*A e2m1*/, 0 /*B e4m3*/, Q, (int)scs[t], Q, (int)bsc[tt]);
         }
     }
-}
-
-struct PfCtx {
-    PfSrc src;
-    const u4v* asp[2];        // weight scale words of the wave's two items
-    const uint8_t* bsp[4];    // activation scale rows of the lane's column in the wave's 4 row tiles
-    int KT, t, bslot, wi, wt, lane;
-};
-
-template <int Q>
-__device__ __forceinline__ void pf_step(const PfCtx& c, PfStage (&st)[2], u4v* lds, int kt, const u4v (&asc)[2],
-                                        const uint32_t (&bsc)[4], v4f (&acc)[2][4][4]) {
-    if (kt >= c.KT) return;
-    if (kt + 2 < c.KT) pf_load(st[Q & 1], c.src, kt + 2);
-    pf_compute<Q>(lds + (Q & 1) * PF_LDS_STAGE, c.wi, c.wt, c.lane, asc, bsc, acc);
-    if (kt + 1 < c.KT) pf_store(st[(Q + 1) & 1], lds + ((Q + 1) & 1) * PF_LDS_STAGE, c.t, c.bslot);
+    __builtin_amdgcn_sched_barrier(0);   // the MFMAs stay in front of the wait: they are what hides the loads
+    pf_wait_fill();
     __syncthreads();
 }
 
+__device__ __forceinline__ void pf_load_scales(const PfCtx& c, int g4, u4v (&asc)[2], uint32_t (&bsc)[4]) {
+    const int g = c.lane >> 4;
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) asc[ii] = c.asp[ii][(size_t)g4 * 64 + c.lane];
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) bsc[tt] = *reinterpret_cast<const uint32_t*>(c.bsp[tt] + g4 * 16 + g * 4);
+}
+
 __device__ __forceinline__ void pf_mainloop(const PfCtx& c, u4v* lds, v4f (&acc)[2][4][4]) {
-    const int KT4 = (c.KT + 3) >> 2, g = c.lane >> 4;
-    PfStage st[2];
-    pf_load(st[0], c.src, 0);
-    if (c.KT > 1) pf_load(st[1], c.src, 1);
+    const int KT4 = (c.KT + 3) >> 2, full = c.KT >> 2;
+    pf_fill(c, lds, 0);
     u4v asc[2], asc_n[2];
     uint32_t bsc[4], bsc_n[4];
-#pragma unroll
-    for (int ii = 0; ii < 2; ++ii) asc[ii] = asc_n[ii] = c.asp[ii][c.lane];
-#pragma unroll
-    for (int tt = 0; tt < 4; ++tt) bsc[tt] = bsc_n[tt] = *reinterpret_cast<const uint32_t*>(c.bsp[tt] + g * 4);
+    pf_load_scales(c, 0, asc, bsc);
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt) acc[ii][t][tt] = (v4f){0.f, 0.f, 0.f, 0.f};
-    pf_store(st[0], lds, c.t, c.bslot);
+    pf_wait_fill();
     __syncthreads();
 #pragma unroll 1
-    for (int g4 = 0; g4 < KT4; ++g4) {
-        if (g4 + 1 < KT4) {
-#pragma unroll
-            for (int ii = 0; ii < 2; ++ii) asc_n[ii] = c.asp[ii][(size_t)(g4 + 1) * 64 + c.lane];
-#pragma unroll
-            for (int tt = 0; tt < 4; ++tt)
-                bsc_n[tt] = *reinterpret_cast<const uint32_t*>(c.bsp[tt] + (g4 + 1) * 16 + g * 4);
-        }
+    for (int g4 = 0; g4 < full; ++g4) {
+        pf_load_scales(c, min(g4 + 1, KT4 - 1), asc_n, bsc_n);
         const int kt = g4 * 4;
-        pf_step<0>(c, st, lds, kt, asc, bsc, acc);
-        pf_step<1>(c, st, lds, kt + 1, asc, bsc, acc);
-        pf_step<2>(c, st, lds, kt + 2, asc, bsc, acc);
-        pf_step<3>(c, st, lds, kt + 3, asc, bsc, acc);
+        pf_step<0>(c, lds, kt, asc, bsc, acc);
+        pf_step<1>(c, lds, kt + 1, asc, bsc, acc);
+        pf_step<2>(c, lds, kt + 2, asc, bsc, acc);
+        pf_step<3>(c, lds, kt + 3, asc, bsc, acc);
 #pragma unroll
         for (int ii = 0; ii < 2; ++ii) asc[ii] = asc_n[ii];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) bsc[tt] = bsc_n[tt];
     }
+    // k steps beyond the last full group of four (block-uniform branches)
+    const int kt = full * 4, rem = c.KT & 3;
+    if (rem > 0) pf_step<0>(c, lds, kt, asc, bsc, acc);
+    if (rem > 1) pf_step<1>(c, lds, kt + 1, asc, bsc, acc);
+    if (rem > 2) pf_step<2>(c, lds, kt + 2, asc, bsc, acc);
 }
 
 // Block -> (unit, item group).  Hardware deals consecutive blocks round-robin over the 8 XCDs; the live work
@@ -481,23 +484,22 @@ __device__ __forceinline__ bool pf_block_work(int n_units, int groups, int& u, i
     return true;
 }
 
-// Fills the block-level part of the context.  row_q(c) returns the e4m3 row of unit column c, row_s(c) its
-// scale row; columns >= nrows alias column 0 (their results are never stored).
+// Fills the context.  row_q(c) returns the e4m3 row of unit column c, row_s(c) its scale row; columns >= nrows
+// alias column 0 (their results are never stored).
 template <typename RowQ, typename RowS>
 __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const uint8_t* sbase, int item0, int items,
                                            int KT, int nrows, RowQ row_q, RowS row_s) {
-    const int t = threadIdx.x, KT4 = (KT + 3) >> 2;
-    c.KT = KT; c.t = t; c.lane = t & 63;
-    const int wave = t >> 6;
-    c.wi = wave & 1; c.wt = wave >> 1;
-    const int j = t & 7, r8 = t >> 3;   // chunk of the k step, row within a group of 32 rows
-    c.bslot = (r8 >> 4) * 128 + (j >> 2) * 64 + (j & 3) * 16 + ((r8 & 15) ^ j);
+    const int KT4 = (KT + 3) >> 2;
+    c.KT = KT;
+    c.lane = threadIdx.x & 63;
+    c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    c.wi = c.wave & 1; c.wt = c.wave >> 1;
+    const int cc = c.lane & 15, g = c.lane >> 4;
+    c.a_src = reinterpret_cast<const u4v*>(cbase) + (size_t)min(item0 + c.wave, items - 1) * KT * 256 + c.lane;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int item = min(item0 + i, items - 1);
-        c.src.a[i] = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256 + t;
-        const int col = r8 + 32 * i;
-        c.src.b[i] = row_q(col < nrows ? col : 0) + j * 16;
+    for (int i = 0; i < 2; ++i) {
+        const int col = (c.wave * 2 + i) * 16 + cc;
+        c.b_src[i] = row_q(col < nrows ? col : 0) + g * 16;
     }
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
@@ -506,12 +508,12 @@ __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const
     }
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
-        const int col = (c.wt * 4 + tt) * 16 + (c.lane & 15);
+        const int col = (c.wt * 4 + tt) * 16 + cc;
         c.bsp[tt] = row_s(col < nrows ? col : 0);
     }
 }
 
-__global__ __launch_bounds__(256) void gate_up_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
+__global__ __launch_bounds__(256, 2) void gate_up_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
                                                               const uint8_t* __restrict__ xs,
                                                               const int32_t* __restrict__ gather_src,
                                                               uint8_t* __restrict__ act_q,
@@ -555,8 +557,8 @@ __global__ __launch_bounds__(256) void gate_up_prefill_kernel(MfmaArgs a, int gr
             float amax = 0.0f;
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                r0[v] = swiglu_ref(acc[ii][0][tt][v], acc[ii][2][tt][v], a.limit);
-                r1[v] = swiglu_ref(acc[ii][1][tt][v], acc[ii][3][tt][v], a.limit);
+                r0[v] = swiglu_fast(acc[ii][0][tt][v], acc[ii][2][tt][v], a.limit);
+                r1[v] = swiglu_fast(acc[ii][1][tt][v], acc[ii][3][tt][v], a.limit);
                 amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
             }
             amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
@@ -564,12 +566,8 @@ __global__ __launch_bounds__(256) void gate_up_prefill_kernel(MfmaArgs a, int gr
             if (col < nrows) {
                 const uint32_t sb = block_scale_e8m0(amax);
                 const float inv = u2f((254u - sb) << 23);
-                uint32_t p0 = 0, p1 = 0;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    p0 |= e4m3_encode(r0[v] * inv) << (8 * v);
-                    p1 |= e4m3_encode(r1[v] * inv) << (8 * v);
-                }
+                const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
+                const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
                 uint8_t* dst = act_q + (size_t)(row0 + col) * a.act_ld + (size_t)item * 32 + g * 4;
                 *reinterpret_cast<uint32_t*>(dst) = p0;
                 *reinterpret_cast<uint32_t*>(dst + 16) = p1;
@@ -579,7 +577,7 @@ __global__ __launch_bounds__(256) void gate_up_prefill_kernel(MfmaArgs a, int gr
     }
 }
 
-__global__ __launch_bounds__(256) void down_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
+__global__ __launch_bounds__(256, 2) void down_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
                                                            const uint8_t* __restrict__ act_s, float* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig;
