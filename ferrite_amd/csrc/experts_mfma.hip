@@ -368,22 +368,26 @@ __device__ __forceinline__ void dma16(const void* g, void* lds_base) {
 
 struct PfCtx {
     const u4v* a_src;         // codes of the item this wave stages, k step 0, + lane
-    const uint8_t* b_src[2];  // e4m3 rows (2*wave+i)*16 + lane%16 of the unit, + 16*(lane/16)
+    const uint8_t* b_src[2];  // e4m3 rows (2*wave+i)*16 + lane/4 of the unit, + the lane's 16-byte chunk
     const u4v* asp[2];        // weight scale words of the wave's two items
     const uint8_t* bsp[4];    // activation scale rows of the lane's column in the wave's 4 row tiles
-    int KT, wave, wi, wt, lane;
+    int KT, wave, wi, wt, lane, bslot;
 };
 
 // Starts the loads of k step kt into `stage`.
 __device__ __forceinline__ void pf_fill(const PfCtx& c, u4v* stage, int kt) {
     const u4v* a = c.a_src + (size_t)kt * 256;
+#ifndef PF_EXP_NOA
 #pragma unroll
     for (int t = 0; t < 4; ++t) dma16(a + t * 64, stage + (c.wave * 4 + t) * 64);
+#endif
+#ifndef PF_EXP_NOB
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
             dma16(c.b_src[i] + (size_t)kt * 128 + h * 64, stage + 1024 + ((c.wave * 2 + i) * 2 + h) * 64);
+#endif
 }
 
 // All loads into LDS issued by this wave have landed (vmcnt 0; expcnt and lgkmcnt left alone).
@@ -400,9 +404,9 @@ __device__ __forceinline__ void pf_step(const PfCtx& c, u4v* lds, int kt, const 
     u4v av[2][4];
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
-        const u4v* bt = cur + 1024 + (c.wt * 4 + tt) * 128;
-        const u4v b0 = bt[c.lane];
-        const u4v b1 = bt[64 + c.lane];
+        const u4v* bt = cur + 1024 + (c.wt * 4 + tt) * 128 + c.bslot;
+        const u4v b0 = bt[0];
+        const u4v b1 = bt[64];
         bv[tt] = (v8i){(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
     }
 #pragma unroll
@@ -410,7 +414,11 @@ __device__ __forceinline__ void pf_step(const PfCtx& c, u4v* lds, int kt, const 
 #pragma unroll
         for (int t = 0; t < 4; ++t) av[ii][t] = cur[((c.wi * 2 + ii) * 4 + t) * 64 + c.lane];
     __builtin_amdgcn_sched_barrier(0);
+#ifdef PF_EXP_HOTLOAD
+    pf_fill(c, lds + ((Q + 1) & 1) * PF_LDS_STAGE, (kt + 1) & 1);
+#else
     pf_fill(c, lds + ((Q + 1) & 1) * PF_LDS_STAGE, min(kt + 1, c.KT - 1));
+#endif
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
@@ -496,11 +504,15 @@ __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const
     c.wi = c.wave & 1; c.wt = c.wave >> 1;
     const int cc = c.lane & 15, g = c.lane >> 4;
     c.a_src = reinterpret_cast<const u4v*>(cbase) + (size_t)min(item0 + c.wave, items - 1) * KT * 256 + c.lane;
+    // Activation stage layout: the four lanes of a quad fetch 64 consecutive bytes of one row (what the texture
+    // addresser coalesces), so row r's 16-byte chunk q of a half k step lands at slot 4r + q; the chunk a lane
+    // fetches is XORed with r/4 so that the operand read of 16 rows at a fixed chunk is spread over all banks.
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int col = (c.wave * 2 + i) * 16 + cc;
-        c.b_src[i] = row_q(col < nrows ? col : 0) + g * 16;
+        const int col = (c.wave * 2 + i) * 16 + (c.lane >> 2);
+        c.b_src[i] = row_q(col < nrows ? col : 0) + ((c.lane & 3) ^ (c.lane >> 4)) * 16;
     }
+    c.bslot = 4 * cc + (g ^ (cc >> 2));
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
         const int item = min(item0 + c.wi * 2 + ii, items - 1);
