@@ -674,10 +674,144 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
     return FERRITE_ERR_INVALID_ARG;
 }
 
+// Router GEMM for many tokens: the same sequential chain (cpu.rs:82-122), register tiled.  A wave owns 64 experts
+// (one per lane, weights from the k-blocked transpose: one coalesced float4 per lane and four k) x T tokens whose
+// activations are wave-uniform and therefore come through scalar loads; every (token, expert) pair still sees
+// acc = acc + x*w for k ascending with separately rounded multiply and add.  T independent chains per lane cover
+// the VALU latency.  grid (Epad/64, ceil(n / (4*T))), 4 waves per block on the same experts.
+// One macro step = KM groups of four k: 16 k for bf16 activations, 8 k for f32, i.e. 32 bytes per token and step.
+template <typename XT>
+struct RouterStep {
+    static constexpr int KM = sizeof(XT) == 4 ? 2 : 4;
+};
+
+template <typename XT, int T, int TE>
+struct RouterSet {
+    uint4 x[T][2];                            // 32 bytes of each token as loaded; wave-uniform -> scalar registers
+    float4 w[RouterStep<XT>::KM][TE];
+};
+
+// Loads only: the bf16 -> f32 shifts happen at the use, so nothing here waits for the data.
+template <typename XT, int T, int TE>
+__device__ __forceinline__ void router_load(RouterSet<XT, T, TE>& r, const XT* const (&xr)[T], const float4* wp,
+                                            int Epad, int step) {
+    constexpr int KM = RouterStep<XT>::KM;
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+        const uint4* p = reinterpret_cast<const uint4*>(xr[i]) + (size_t)step * 2;
+        r.x[i][0] = p[0];
+        r.x[i][1] = p[1];
+    }
+#pragma unroll
+    for (int q = 0; q < KM; ++q)
+#pragma unroll
+        for (int j = 0; j < TE; ++j) r.w[q][j] = wp[(size_t)(step * KM + q) * Epad + j * 64];
+}
+
+template <typename XT, int T, int TE>
+__device__ __forceinline__ void router_chain(float (&acc)[TE][T], const RouterSet<XT, T, TE>& r) {
+    constexpr int KM = RouterStep<XT>::KM;
+#pragma unroll
+    for (int q = 0; q < KM; ++q) {
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+            float x0, x1, x2, x3;
+            if constexpr (sizeof(XT) == 4) {
+                const uint4 v = r.x[i][q];
+                x0 = u2f(v.x); x1 = u2f(v.y); x2 = u2f(v.z); x3 = u2f(v.w);
+            } else {
+                const uint4 v = r.x[i][q >> 1];
+                const uint32_t lo = (q & 1) ? v.z : v.x, hi = (q & 1) ? v.w : v.y;
+                x0 = u2f(lo << 16); x1 = u2f(lo & 0xffff0000u); x2 = u2f(hi << 16); x3 = u2f(hi & 0xffff0000u);
+            }
+#pragma unroll
+            for (int j = 0; j < TE; ++j) {
+                float a = acc[j][i];
+                a = fadd(a, fmul(x0, r.w[q][j].x));
+                a = fadd(a, fmul(x1, r.w[q][j].y));
+                a = fadd(a, fmul(x2, r.w[q][j].z));
+                a = fadd(a, fmul(x3, r.w[q][j].w));
+                acc[j][i] = a;
+            }
+        }
+    }
+}
+
+// TE blocks of 64 experts (lane = expert within the block) x T tokens per wave.
+template <typename XT, int T, int TE>
+__global__ __launch_bounds__(256) void router_tile_kernel(const XT* __restrict__ x, const float4* __restrict__ wt,
+                                                          int n, int H, int E, int Epad, float* __restrict__ logits) {
+    constexpr int KM = RouterStep<XT>::KM;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t0 = (blockIdx.y * 4 + wave) * T;
+    if (t0 >= n) return;
+    const int e0 = blockIdx.x * 64 * TE + lane;
+    const float4* wp = wt + e0;
+    const XT* xr[T];
+#pragma unroll
+    for (int i = 0; i < T; ++i) xr[i] = x + (size_t)min(t0 + i, n - 1) * H;
+    float acc[TE][T];
+#pragma unroll
+    for (int j = 0; j < TE; ++j)
+#pragma unroll
+        for (int i = 0; i < T; ++i) acc[j][i] = 0.0f;
+    const int nsteps = H / (4 * KM);   // even: H % 128 == 0
+    RouterSet<XT, T, TE> sa, sb;
+    router_load(sa, xr, wp, Epad, 0);
+    // Two register sets alternate: the loads of one are issued before the chains over the other.  Scalar loads
+    // return out of order, so any wait on them is a wait for all of them: the set about to be used is waited
+    // for BEFORE the other set's loads are issued (0xC07F: lgkmcnt 0, vmcnt and expcnt untouched).
+    for (int st = 0; st < nsteps; st += 2) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        router_load(sb, xr, wp, Epad, st + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        router_chain(acc, sa);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        router_load(sa, xr, wp, Epad, min(st + 2, nsteps - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        router_chain(acc, sb);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int j = 0; j < TE; ++j) {
+        const int e = e0 + j * 64;
+        if (e < E) {
+#pragma unroll
+            for (int i = 0; i < T; ++i)
+                if (t0 + i < n) logits[(size_t)(t0 + i) * E + e] = acc[j][i];
+        }
+    }
+}
+
+template <typename XT>
+static int launch_router_tile(const void* x, const float* router_t, int n, int H, int E, float* logits, hipStream_t st) {
+    const int Epad = (E + 63) / 64 * 64;
+    const XT* xp = static_cast<const XT*>(x);
+    const float4* wp = reinterpret_cast<const float4*>(router_t);
+    constexpr int T = 4;
+    dim3 grid(1, (n + 4 * T - 1) / (4 * T));
+    // two expert blocks per wave halve the weight traffic, but only when enough waves remain to hide latency
+    if (Epad % 128 == 0 && (long)(Epad / 128) * grid.y * 4 >= 4096) {
+        grid.x = Epad / 128;
+        router_tile_kernel<XT, T, 2><<<grid, 256, 0, st>>>(xp, wp, n, H, E, Epad, logits);
+    } else {
+        grid.x = Epad / 64;
+        router_tile_kernel<XT, T, 1><<<grid, 256, 0, st>>>(xp, wp, n, H, E, Epad, logits);
+    }
+    return check_launch("router_tile");
+}
+
 // Router GEMM alone from the transposed weight (any n): logits only.
 int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
                         hipStream_t st) {
     if (H % 128 != 0 || n <= 0 || (size_t)H * 4 > 60 * 1024 || n > 65535) return FERRITE_DECLINED;
+    if (n >= 64) {
+        if (x_dtype == FERRITE_DT_F32) return launch_router_tile<float>(x, router_t, n, H, E, logits, st);
+        if (x_dtype == FERRITE_DT_BF16) return launch_router_tile<uint16_t>(x, router_t, n, H, E, logits, st);
+        return FERRITE_ERR_INVALID_ARG;
+    }
     HeadArgs a{};
     a.x = x; a.wt = router_t; a.n = n; a.H = H; a.E = E; a.Epad = (E + 63) / 64 * 64; a.logits = logits;
     dim3 grid(a.Epad / 64, n);
