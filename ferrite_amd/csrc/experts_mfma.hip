@@ -660,19 +660,6 @@ static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int
     return a;
 }
 
-// Kernels that need more than 64 KiB of dynamic LDS must have the limit raised once (a function attribute,
-// not a stream operation).  `raised` remembers the largest value already set for that kernel.
-template <typename K>
-static int set_lds_limit(K kernel, size_t bytes, size_t* raised) {
-    if (bytes <= 64 * 1024 || bytes <= *raised) return FERRITE_OK;
-    if (bytes > 160 * 1024) return FERRITE_DECLINED;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-    *raised = bytes;
-    return FERRITE_OK;
-}
-
 int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
                         int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
                         hipStream_t st) {

@@ -38,6 +38,19 @@ inline int max_units_for(int n, int topk, int n_experts, int has_shared, int uni
 // variable FERRITE_HIP_UNIT_ROWS (16 or 128) overrides the choice; it is read at every call.
 int unit_rows_for(int n, int topk, int n_experts);
 
+// Kernels that need more than 64 KiB of dynamic LDS must have the limit raised once (a function attribute,
+// not a stream operation).  `raised` remembers the largest value already set for that kernel.
+template <typename K>
+inline int set_lds_limit(K kernel, size_t bytes, size_t* raised) {
+    if (bytes <= 64 * 1024 || bytes <= *raised) return FERRITE_OK;
+    if (bytes > 160 * 1024) return FERRITE_DECLINED;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+    *raised = bytes;
+    return FERRITE_OK;
+}
+
 // route.hip
 int launch_matmul_exact(const void* x, int x_dtype, const float* w, const float* bias, float* out, int n, int k,
                         int o, hipStream_t st);

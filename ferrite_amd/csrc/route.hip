@@ -506,20 +506,25 @@ __global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const 
 
 // ------------------------------------------------------------------------------------------------
 // The head of the layer as ONE launch (decode-sized batches), or the router GEMM alone (kFused = false).
-// Every workgroup is a single wave.
-//   blocks (eb, t), eb < eblocks : router logits of token t for experts [64 eb, 64 eb + 64), one lane per
-//                                  expert: the reference's sequential chain.  The router weight comes from its
-//                                  k-blocked transpose [H/4][Epad][4], so the wave's load for four k is one
-//                                  contiguous 1 KiB; two register sets of 16 such loads alternate (the loads
-//                                  of one set fly while the chain consumes the other); x[t] sits in LDS as f32
+// Workgroups have four waves.
+//   blocks (eb, t), eb < eblocks : router logits of token t for experts [64 eb, 64 eb + 64): the reference's
+//                                  sequential chain, one lane of wave 0 per expert.  A lone wave issues one
+//                                  instruction every four cycles, loads and address arithmetic included, so the
+//                                  chain wave is left with nothing but the adds: waves 1-3 fetch the router
+//                                  weight (k-blocked transpose [H/4][Epad][4], four chunks ahead), multiply it
+//                                  with x[t] (the products are order-independent and each rounded once, as in
+//                                  the reference) and hand the products over through a two-buffer LDS ring of
+//                                  32-group chunks; wave 0 reads them back and adds them in k order
 //   blocks (eblocks, t)          : e4m3-per-32 quantisation of x[t] (off the critical path)
-//   last logits wave of a token  : routes the token (arrival counter per token)
+//   last logits block of a token : its wave 0 routes the token (arrival counter per token)
 //   last routed token            : builds the permutation and unit tables, then clears the counters so the
 //                                  next launch (or graph replay) starts clean
 // counters[0] = routed tokens, counters[1 + t] = logits blocks of token t that have arrived; all zero on entry.
 // ------------------------------------------------------------------------------------------------
 constexpr int HEAD_MAX_N = 256;
-constexpr int HD_D = 16;   // float4 loads per register set
+constexpr int HD_CH = 32;                              // groups of four k per chunk
+constexpr int HD_PW = (HD_CH + 2) / 3;                 // groups per producer wave and chunk (11, 11, 10)
+constexpr size_t HD_RING_BYTES = 2 * (size_t)HD_CH * 1024;
 
 struct HeadArgs {
     const void* x;
@@ -535,47 +540,133 @@ struct HeadArgs {
 };
 
 struct HeadSet {
-    float4 w[HD_D];
+    float4 w[HD_PW];
 };
 
-__device__ __forceinline__ void head_load(HeadSet& st, const char* __restrict__ base, unsigned ldb, unsigned loff,
-                                          int k0, int nk4) {
+// Producer P (0..2) owns groups P, P+3, ... of every chunk.  Chunks past the end re-read the last one (never
+// consumed), which keeps every load unconditional.
+template <int P>
+__device__ __forceinline__ void head_pload(HeadSet& st, const float4* __restrict__ wp, int Epad, int c, int nch) {
+    const float4* base = wp + (size_t)min(c, nch - 1) * HD_CH * Epad;
 #pragma unroll
-    for (int j = 0; j < HD_D; ++j) {
-        const int kn = min(k0 + j, nk4 - 1);   // past the end: a valid row that is never used
-        st.w[j] = *reinterpret_cast<const float4*>(base + (size_t)kn * ldb + loff);
+    for (int i = 0; i < HD_PW; ++i)
+        if (P + 3 * i < HD_CH) st.w[i] = base[(size_t)(P + 3 * i) * Epad];
+}
+
+template <int P>
+__device__ __forceinline__ void head_pmul(const HeadSet& st, const float4* xc, float4* buf, int lane) {
+#pragma unroll
+    for (int i = 0; i < HD_PW; ++i) {
+        const int j = P + 3 * i;
+        if (j < HD_CH) {
+            const float4 xv = xc[j], wv = st.w[i];
+            buf[j * 64 + lane] = make_float4(fmul(xv.x, wv.x), fmul(xv.y, wv.y), fmul(xv.z, wv.z), fmul(xv.w, wv.w));
+        }
     }
 }
 
-__device__ __forceinline__ float head_chain(float s, const HeadSet& st, const float4* xl) {
+// Products of chunk c+1 are made while the chain consumes chunk c; register set c%4 holds the weights of chunk c
+// and is reloaded for chunk c+4 as soon as it has been used.
+template <int P>
+__device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int Epad, int nch, const float4* xl,
+                                              float4* ring, int lane) {
+    float4* b0 = ring;
+    float4* b1 = ring + HD_CH * 64;
+    HeadSet s0, s1, s2, s3;
+    head_pload<P>(s0, wp, Epad, 0, nch);
+    head_pload<P>(s1, wp, Epad, 1, nch);
+    head_pload<P>(s2, wp, Epad, 2, nch);
+    head_pload<P>(s3, wp, Epad, 3, nch);
+    __syncthreads();   // x[t] is in LDS
+    head_pmul<P>(s0, xl, b0, lane);
+    head_pload<P>(s0, wp, Epad, 4, nch);
+    __syncthreads();
+    for (int c = 0; c < nch; c += 4) {
+        head_pmul<P>(s1, xl + min(c + 1, nch - 1) * HD_CH, b1, lane);
+        head_pload<P>(s1, wp, Epad, c + 5, nch);
+        __syncthreads();
+        head_pmul<P>(s2, xl + min(c + 2, nch - 1) * HD_CH, b0, lane);
+        head_pload<P>(s2, wp, Epad, c + 6, nch);
+        __syncthreads();
+        head_pmul<P>(s3, xl + min(c + 3, nch - 1) * HD_CH, b1, lane);
+        head_pload<P>(s3, wp, Epad, c + 7, nch);
+        __syncthreads();
+        head_pmul<P>(s0, xl + min(c + 4, nch - 1) * HD_CH, b0, lane);
+        head_pload<P>(s0, wp, Epad, c + 8, nch);
+        __syncthreads();
+    }
+}
+
+// The chain over one chunk of products: batches of eight LDS reads, one wait per batch (0xC87F: lgkmcnt <= 8, i.e.
+// everything but the batch just issued; 0xC07F: lgkmcnt 0), 32 dependent adds per batch.
+__device__ __forceinline__ float head_consume(float s, const float4* buf, int lane) {
+    float4 r[2][8];
 #pragma unroll
-    for (int j = 0; j < HD_D; ++j) {
-        const float4 xv = xl[j], wv = st.w[j];
-        s = fadd(s, fmul(xv.x, wv.x));
-        s = fadd(s, fmul(xv.y, wv.y));
-        s = fadd(s, fmul(xv.z, wv.z));
-        s = fadd(s, fmul(xv.w, wv.w));
+    for (int j = 0; j < 8; ++j) r[0][j] = buf[j * 64 + lane];
+#pragma unroll
+    for (int g = 0; g < HD_CH / 8; ++g) {
+        if (g + 1 < HD_CH / 8) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) r[(g + 1) & 1][j] = buf[((g + 1) * 8 + j) * 64 + lane];
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xC87F);
+        } else {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float4 p = r[g & 1][j];
+            s = fadd(s, p.x);
+            s = fadd(s, p.y);
+            s = fadd(s, p.z);
+            s = fadd(s, p.w);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    return s;
+}
+
+// Barriers pair one to one with head_producer's.
+__device__ __forceinline__ float head_consumer(int nch, const float4* ring, int lane) {
+    const float4* b0 = ring;
+    const float4* b1 = ring + HD_CH * 64;
+    float s = 0.0f;
+    __syncthreads();
+    __syncthreads();
+    for (int c = 0; c < nch; c += 4) {
+        s = head_consume(s, b0, lane);
+        __syncthreads();
+        if (c + 1 < nch) s = head_consume(s, b1, lane);
+        __syncthreads();
+        if (c + 2 < nch) s = head_consume(s, b0, lane);
+        __syncthreads();
+        if (c + 3 < nch) s = head_consume(s, b1, lane);
+        __syncthreads();
     }
     return s;
 }
 
 template <typename XT, bool kFused>
-__global__ __launch_bounds__(64) void moe_head_kernel(HeadArgs a) {
+__global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
     extern __shared__ __align__(16) unsigned char head_lds[];
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int eb = blockIdx.x, t = blockIdx.y;
     const int eblocks = a.Epad >> 6;
     const int H = a.H;
     const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
     if (eb == eblocks) {
-        for (int b = lane; b < H / 32; b += 64)
+        for (int b = tid; b < H / 32; b += 256)
             a.xs[(size_t)t * scale_pitch(H) + scale_pos(b)] =
                 (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
         return;
     }
-    float4* xl = reinterpret_cast<float4*>(head_lds);
-    const int nk4 = H / 4;   // a multiple of 2 * HD_D (H % 128 == 0)
-    for (int i = lane; i < nk4; i += 64) {
+    float4* ring = reinterpret_cast<float4*>(head_lds);
+    float4* xl = reinterpret_cast<float4*>(head_lds + HD_RING_BYTES);
+    const int nk4 = H / 4, nch = nk4 / HD_CH;   // H % 128 == 0
+    const float4* wp = reinterpret_cast<const float4*>(a.wt) + (size_t)eb * 64 + lane;
+    for (int i = tid; i < nk4; i += 256) {
         float4 v;
         if constexpr (sizeof(XT) == 4) {
             v = reinterpret_cast<const float4*>(xrow)[i];
@@ -585,23 +676,12 @@ __global__ __launch_bounds__(64) void moe_head_kernel(HeadArgs a) {
         }
         xl[i] = v;
     }
-    const char* base = reinterpret_cast<const char*>(a.wt) + (size_t)eb * 64 * 16;
-    const unsigned ldb = (unsigned)a.Epad * 16, loff = (unsigned)lane * 16;
-    HeadSet sa, sb;
-    head_load(sa, base, ldb, loff, 0, nk4);
-    __syncthreads();
     float s = 0.0f;
-    // the scheduling barriers pin "issue one set's loads, then chain over the other set"
-    for (int kk = 0; kk < nk4; kk += 2 * HD_D) {
-        head_load(sb, base, ldb, loff, kk + HD_D, nk4);
-        __builtin_amdgcn_sched_barrier(0);
-        s = head_chain(s, sa, xl + kk);
-        __builtin_amdgcn_sched_barrier(0);
-        head_load(sa, base, ldb, loff, kk + 2 * HD_D, nk4);
-        __builtin_amdgcn_sched_barrier(0);
-        s = head_chain(s, sb, xl + kk + HD_D);
-        __builtin_amdgcn_sched_barrier(0);
-    }
+    if (wave == 0) s = head_consumer(nch, ring, lane);
+    else if (wave == 1) head_producer<0>(wp, a.Epad, nch, xl, ring, lane);
+    else if (wave == 2) head_producer<1>(wp, a.Epad, nch, xl, ring, lane);
+    else head_producer<2>(wp, a.Epad, nch, xl, ring, lane);
+    if (wave != 0) return;   // from here on the block is wave 0 alone; LDS is free for the scratch below
     const int e = eb * 64 + lane;
     if (e < a.E) a.logits[(size_t)t * a.E + e] = s;
     if constexpr (!kFused) return;
@@ -613,7 +693,7 @@ __global__ __launch_bounds__(64) void moe_head_kernel(HeadArgs a) {
     last = __shfl(last, 0, 64);
     if (!last) return;
     __threadfence();
-    __syncthreads();   // x in LDS is dead from here; the scratch below aliases it
+    wave_sync();
     RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds);
     route_wave<true>(a.logits + (size_t)t * a.E, a.bias, true, a.E, a.topk, a.n_group, a.topk_group, a.scaling, sc,
                      a.probs + (size_t)t * a.topk, a.ids_f32 + (size_t)t * a.topk, a.ids + (size_t)t * a.topk);
@@ -623,13 +703,13 @@ __global__ __launch_bounds__(64) void moe_head_kernel(HeadArgs a) {
     last = __shfl(last, 0, 64);
     if (!last) return;
     __threadfence();
-    __syncthreads();
+    wave_sync();
     permute_in_block<true, true>(a.perm, reinterpret_cast<unsigned long long*>(head_lds));
     for (int i = lane; i < a.n + 1; i += 64) a.counters[i] = 0;
 }
 
 static size_t head_lds_bytes(int n, int H, int E, bool fused) {
-    size_t b = (size_t)H * 4;
+    size_t b = HD_RING_BYTES + (size_t)H * 4;
     if (fused) {
         if (b < sizeof(RouteScratch)) b = sizeof(RouteScratch);
         size_t p = perm_block_lds_bytes(n, E);
@@ -639,12 +719,15 @@ static size_t head_lds_bytes(int n, int H, int E, bool fused) {
 }
 
 bool head_supported(int n, int H, int E) {
-    return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, H, E, true) <= 60 * 1024;
+    return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, H, E, true) <= 160 * 1024;
 }
 
 template <typename XT, bool kFused>
 static int launch_head_t(const HeadArgs& a, dim3 grid, size_t lds, hipStream_t st) {
-    moe_head_kernel<XT, kFused><<<grid, 64, lds, st>>>(a);
+    static size_t raised = 0;
+    int rc = set_lds_limit(moe_head_kernel<XT, kFused>, lds, &raised);
+    if (rc) return rc;
+    moe_head_kernel<XT, kFused><<<grid, 256, lds, st>>>(a);
     return check_launch("moe_head");
 }
 
@@ -806,12 +889,13 @@ static int launch_router_tile(const void* x, const float* router_t, int n, int H
 // Router GEMM alone from the transposed weight (any n): logits only.
 int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
                         hipStream_t st) {
-    if (H % 128 != 0 || n <= 0 || (size_t)H * 4 > 60 * 1024 || n > 65535) return FERRITE_DECLINED;
+    if (H % 128 != 0 || n <= 0 || n > 65535) return FERRITE_DECLINED;
     if (n >= 64) {
         if (x_dtype == FERRITE_DT_F32) return launch_router_tile<float>(x, router_t, n, H, E, logits, st);
         if (x_dtype == FERRITE_DT_BF16) return launch_router_tile<uint16_t>(x, router_t, n, H, E, logits, st);
         return FERRITE_ERR_INVALID_ARG;
     }
+    if (head_lds_bytes(n, H, E, false) > 160 * 1024) return FERRITE_DECLINED;
     HeadArgs a{};
     a.x = x; a.wt = router_t; a.n = n; a.H = H; a.E = E; a.Epad = (E + 63) / 64 * 64; a.logits = logits;
     dim3 grid(a.Epad / 64, n);
