@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int j = 0; j < topk; ++j) {
         int g = perm_map[(size_t)t * topk + j];
-        if (g < 0) continue;
+        if (g < 0 || g >= n * topk) continue;   // tables of an uninitialised workspace must not cause a fault
         float p = probs[(size_t)t * topk + j];
         float4 v = *reinterpret_cast<const float4*>(y + (size_t)g * H + h);
         o.x = fadd(o.x, fmul(p, v.x)); o.y = fadd(o.y, fmul(p, v.y));

@@ -506,11 +506,11 @@ __global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const 
 
 // ------------------------------------------------------------------------------------------------
 // The head of the layer as ONE launch (decode-sized batches), or the router GEMM alone (kFused = false).
-// Workgroups have four waves.
+// Workgroups have eight waves.
 //   blocks (eb, t), eb < eblocks : router logits of token t for experts [64 eb, 64 eb + 64): the reference's
 //                                  sequential chain, one lane of wave 0 per expert.  A lone wave issues one
 //                                  instruction every four cycles, loads and address arithmetic included, so the
-//                                  chain wave is left with nothing but the adds: waves 1-3 fetch the router
+//                                  chain wave is left with nothing but the adds: six producer waves fetch the router
 //                                  weight (k-blocked transpose [H/4][Epad][4], four chunks ahead), multiply it
 //                                  with x[t] (the products are order-independent and each rounded once, as in
 //                                  the reference) and hand the products over through a two-buffer LDS ring of
@@ -523,7 +523,8 @@ __global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const 
 // ------------------------------------------------------------------------------------------------
 constexpr int HEAD_MAX_N = 256;
 constexpr int HD_CH = 32;                              // groups of four k per chunk
-constexpr int HD_PW = (HD_CH + 2) / 3;                 // groups per producer wave and chunk (11, 11, 10)
+constexpr int HD_NP = 6;                               // producer waves
+constexpr int HD_PW = (HD_CH + HD_NP - 1) / HD_NP;     // groups per producer wave and chunk (6 or 5)
 constexpr size_t HD_RING_BYTES = 2 * (size_t)HD_CH * 1024;
 
 struct HeadArgs {
@@ -543,21 +544,24 @@ struct HeadSet {
     float4 w[HD_PW];
 };
 
-// Producer P (0..2) owns groups P, P+3, ... of every chunk.  Chunks past the end re-read the last one (never
+// Producer P (0..HD_NP-1) owns groups P, P+HD_NP, ... of every chunk.  Chunks past the end re-read the last one (never
 // consumed), which keeps every load unconditional.
 template <int P>
 __device__ __forceinline__ void head_pload(HeadSet& st, const float4* __restrict__ wp, int Epad, int c, int nch) {
     const float4* base = wp + (size_t)min(c, nch - 1) * HD_CH * Epad;
 #pragma unroll
     for (int i = 0; i < HD_PW; ++i)
-        if (P + 3 * i < HD_CH) st.w[i] = base[(size_t)(P + 3 * i) * Epad];
+        if (P + HD_NP * i < HD_CH) st.w[i] = base[(size_t)(P + HD_NP * i) * Epad];
 }
 
 template <int P>
 __device__ __forceinline__ void head_pmul(const HeadSet& st, const float4* xc, float4* buf, int lane) {
+#ifdef HD_EXP_NOPROD
+    return;
+#endif
 #pragma unroll
     for (int i = 0; i < HD_PW; ++i) {
-        const int j = P + 3 * i;
+        const int j = P + HD_NP * i;
         if (j < HD_CH) {
             const float4 xv = xc[j], wv = st.w[i];
             buf[j * 64 + lane] = make_float4(fmul(xv.x, wv.x), fmul(xv.y, wv.y), fmul(xv.z, wv.z), fmul(xv.w, wv.w));
@@ -600,6 +604,9 @@ __device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int
 // The chain over one chunk of products: batches of eight LDS reads, one wait per batch (0xC87F: lgkmcnt <= 8, i.e.
 // everything but the batch just issued; 0xC07F: lgkmcnt 0), 32 dependent adds per batch.
 __device__ __forceinline__ float head_consume(float s, const float4* buf, int lane) {
+#ifdef HD_EXP_NOCONS
+    return s;
+#endif
     float4 r[2][8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) r[0][j] = buf[j * 64 + lane];
@@ -648,7 +655,7 @@ __device__ __forceinline__ float head_consumer(int nch, const float4* ring, int 
 }
 
 template <typename XT, bool kFused>
-__global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
+__global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
     extern __shared__ __align__(16) unsigned char head_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -657,7 +664,7 @@ __global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
     const int H = a.H;
     const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
     if (eb == eblocks) {
-        for (int b = tid; b < H / 32; b += 256)
+        for (int b = tid; b < H / 32; b += 512)
             a.xs[(size_t)t * scale_pitch(H) + scale_pos(b)] =
                 (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
         return;
@@ -666,7 +673,7 @@ __global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
     float4* xl = reinterpret_cast<float4*>(head_lds + HD_RING_BYTES);
     const int nk4 = H / 4, nch = nk4 / HD_CH;   // H % 128 == 0
     const float4* wp = reinterpret_cast<const float4*>(a.wt) + (size_t)eb * 64 + lane;
-    for (int i = tid; i < nk4; i += 256) {
+    for (int i = tid; i < nk4; i += 512) {
         float4 v;
         if constexpr (sizeof(XT) == 4) {
             v = reinterpret_cast<const float4*>(xrow)[i];
@@ -676,11 +683,18 @@ __global__ __launch_bounds__(256) void moe_head_kernel(HeadArgs a) {
         }
         xl[i] = v;
     }
+    // wave 0 chains; wave 4 would share its SIMD (and its VALU issue slots) and leaves; the others produce
     float s = 0.0f;
-    if (wave == 0) s = head_consumer(nch, ring, lane);
-    else if (wave == 1) head_producer<0>(wp, a.Epad, nch, xl, ring, lane);
-    else if (wave == 2) head_producer<1>(wp, a.Epad, nch, xl, ring, lane);
-    else head_producer<2>(wp, a.Epad, nch, xl, ring, lane);
+    switch (wave) {
+        case 0: s = head_consumer(nch, ring, lane); break;
+        case 1: head_producer<0>(wp, a.Epad, nch, xl, ring, lane); break;
+        case 2: head_producer<1>(wp, a.Epad, nch, xl, ring, lane); break;
+        case 3: head_producer<2>(wp, a.Epad, nch, xl, ring, lane); break;
+        case 5: head_producer<3>(wp, a.Epad, nch, xl, ring, lane); break;
+        case 6: head_producer<4>(wp, a.Epad, nch, xl, ring, lane); break;
+        case 7: head_producer<5>(wp, a.Epad, nch, xl, ring, lane); break;
+        default: __syncthreads(); break;   // its share of x[t] is in LDS before it goes
+    }
     if (wave != 0) return;   // from here on the block is wave 0 alone; LDS is free for the scratch below
     const int e = eb * 64 + lane;
     if (e < a.E) a.logits[(size_t)t * a.E + e] = s;
@@ -727,7 +741,7 @@ static int launch_head_t(const HeadArgs& a, dim3 grid, size_t lds, hipStream_t s
     static size_t raised = 0;
     int rc = set_lds_limit(moe_head_kernel<XT, kFused>, lds, &raised);
     if (rc) return rc;
-    moe_head_kernel<XT, kFused><<<grid, 256, lds, st>>>(a);
+    moe_head_kernel<XT, kFused><<<grid, 512, lds, st>>>(a);
     return check_launch("moe_head");
 }
 
