@@ -377,17 +377,13 @@ struct PfCtx {
 // Starts the loads of k step kt into `stage`.
 __device__ __forceinline__ void pf_fill(const PfCtx& c, u4v* stage, int kt) {
     const u4v* a = c.a_src + (size_t)kt * 256;
-#ifndef PF_EXP_NOA
 #pragma unroll
     for (int t = 0; t < 4; ++t) dma16(a + t * 64, stage + (c.wave * 4 + t) * 64);
-#endif
-#ifndef PF_EXP_NOB
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
             dma16(c.b_src[i] + (size_t)kt * 128 + h * 64, stage + 1024 + ((c.wave * 2 + i) * 2 + h) * 64);
-#endif
 }
 
 // All loads into LDS issued by this wave have landed (vmcnt 0; expcnt and lgkmcnt left alone).
@@ -414,11 +410,7 @@ __device__ __forceinline__ void pf_step(const PfCtx& c, u4v* lds, int kt, const 
 #pragma unroll
         for (int t = 0; t < 4; ++t) av[ii][t] = cur[((c.wi * 2 + ii) * 4 + t) * 64 + c.lane];
     __builtin_amdgcn_sched_barrier(0);
-#ifdef PF_EXP_HOTLOAD
-    pf_fill(c, lds + ((Q + 1) & 1) * PF_LDS_STAGE, (kt + 1) & 1);
-#else
     pf_fill(c, lds + ((Q + 1) & 1) * PF_LDS_STAGE, min(kt + 1, c.KT - 1));
-#endif
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
@@ -558,14 +550,6 @@ __global__ __launch_bounds__(256, 2) void gate_up_prefill_kernel(MfmaArgs a, int
 
     const int cc = c.lane & 15, g = c.lane >> 4;
     const int apitch = scale_pitch(a.act_ld);
-#ifdef PF_EXP_NOEPI
-    if (a.limit == 12345.f) {
-        float sum = 0.f;
-        for (int ii = 0; ii < 2; ++ii) for (int t = 0; t < 4; ++t) for (int tt = 0; tt < 4; ++tt) for (int v = 0; v < 4; ++v) sum += acc[ii][t][tt][v];
-        act_q[threadIdx.x] = (uint8_t)sum;
-    }
-    return;
-#endif
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
         const int item = item0 + c.wi * 2 + ii;

@@ -193,17 +193,18 @@ __device__ __forceinline__ void wave_sync() {
 
 // One wave routes one token.  `lg` = the token's e logits.  The scratch is private to the wave, so waves of
 // a block may call this independently of each other.
-template <bool kCoherent>
-__device__ __forceinline__ void route_wave(const float* __restrict__ lg, const float* __restrict__ bias, bool live,
+// NI = expert slots per lane (ceil(e / 64) rounded up to 1, 2, 4 or 8): everything below costs in proportion to it.
+template <bool kCoherent, int NI>
+__device__ __forceinline__ void route_wave_ni(const float* __restrict__ lg, const float* __restrict__ bias, bool live,
                                            int e, int topk, int n_group, int topk_group, float scaling,
                                            RouteScratch& sc, float* __restrict__ probs, float* __restrict__ ids_f32,
                                            int32_t* __restrict__ ids_i32) {
     const int lane = threadIdx.x & 63;
     const int ni = (e + 63) >> 6;
-    float sg[RT_NI], ch[RT_NI];
-    bool ok[RT_NI];
+    float sg[NI], ch[NI];
+    bool ok[NI];
 #pragma unroll
-    for (int i = 0; i < RT_NI; ++i) {
+    for (int i = 0; i < NI; ++i) {
         int j = lane + 64 * i;
         ok[i] = live && i < ni && j < e;
         float l = 0.0f;
@@ -216,7 +217,7 @@ __device__ __forceinline__ void route_wave(const float* __restrict__ lg, const f
     if (n_group > 1) {
         const int gs = e / n_group;
 #pragma unroll
-        for (int i = 0; i < RT_NI; ++i) {
+        for (int i = 0; i < NI; ++i) {
             int j = lane + 64 * i;
             if (i < ni && j < e) sc.choice[j] = ch[i];
         }
@@ -241,31 +242,31 @@ __device__ __forceinline__ void route_wave(const float* __restrict__ lg, const f
         if (lane < n_group) sc.keep[lane] = rank < topk_group ? 1 : 0;
         wave_sync();
 #pragma unroll
-        for (int i = 0; i < RT_NI; ++i) {
+        for (int i = 0; i < NI; ++i) {
             int j = lane + 64 * i;
             if (ok[i] && !sc.keep[j / gs]) ok[i] = false;
         }
     }
 
     // key = (order-preserving bits of choice, inverted index): larger key = earlier in the reference's sort
-    unsigned long long key[RT_NI];
+    unsigned long long key[NI];
 #pragma unroll
-    for (int i = 0; i < RT_NI; ++i) {
+    for (int i = 0; i < NI; ++i) {
         uint32_t j = lane + 64 * i;
         key[i] = ok[i] ? (((unsigned long long)ordered_u32(ch[i]) << 32) | (0xFFFFFFFFu - j)) : 0ull;
         if (i < ni && (int)j < e) sc.key[j] = key[i];
     }
     wave_sync();
-    int rank[RT_NI];
+    int rank[NI];
 #pragma unroll
-    for (int i = 0; i < RT_NI; ++i) rank[i] = 0;
+    for (int i = 0; i < NI; ++i) rank[i] = 0;
     for (int j2 = 0; j2 < e; ++j2) {
         const unsigned long long kj = sc.key[j2];   // same address in every lane: an LDS broadcast
 #pragma unroll
-        for (int i = 0; i < RT_NI; ++i) rank[i] += kj > key[i] ? 1 : 0;
+        for (int i = 0; i < NI; ++i) rank[i] += kj > key[i] ? 1 : 0;
     }
 #pragma unroll
-    for (int i = 0; i < RT_NI; ++i) {
+    for (int i = 0; i < NI; ++i) {
         if (key[i] != 0ull && rank[i] < topk) {
             sc.sel_id[rank[i]] = lane + 64 * i;
             sc.sel_sig[rank[i]] = sg[i];
@@ -282,6 +283,17 @@ __device__ __forceinline__ void route_wave(const float* __restrict__ lg, const f
         if (ids_f32) ids_f32[lane] = (float)my_id;
         if (ids_i32) ids_i32[lane] = my_id;
     }
+}
+
+template <bool kCoherent>
+__device__ __forceinline__ void route_wave(const float* __restrict__ lg, const float* __restrict__ bias, bool live,
+                                           int e, int topk, int n_group, int topk_group, float scaling,
+                                           RouteScratch& sc, float* __restrict__ probs, float* __restrict__ ids_f32,
+                                           int32_t* __restrict__ ids_i32) {
+    if (e <= 64) route_wave_ni<kCoherent, 1>(lg, bias, live, e, topk, n_group, topk_group, scaling, sc, probs, ids_f32, ids_i32);
+    else if (e <= 128) route_wave_ni<kCoherent, 2>(lg, bias, live, e, topk, n_group, topk_group, scaling, sc, probs, ids_f32, ids_i32);
+    else if (e <= 256) route_wave_ni<kCoherent, 4>(lg, bias, live, e, topk, n_group, topk_group, scaling, sc, probs, ids_f32, ids_i32);
+    else route_wave_ni<kCoherent, 8>(lg, bias, live, e, topk, n_group, topk_group, scaling, sc, probs, ids_f32, ids_i32);
 }
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits,
@@ -556,9 +568,6 @@ __device__ __forceinline__ void head_pload(HeadSet& st, const float4* __restrict
 
 template <int P>
 __device__ __forceinline__ void head_pmul(const HeadSet& st, const float4* xc, float4* buf, int lane) {
-#ifdef HD_EXP_NOPROD
-    return;
-#endif
 #pragma unroll
     for (int i = 0; i < HD_PW; ++i) {
         const int j = P + HD_NP * i;
@@ -604,9 +613,6 @@ __device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int
 // The chain over one chunk of products: batches of eight LDS reads, one wait per batch (0xC87F: lgkmcnt <= 8, i.e.
 // everything but the batch just issued; 0xC07F: lgkmcnt 0), 32 dependent adds per batch.
 __device__ __forceinline__ float head_consume(float s, const float4* buf, int lane) {
-#ifdef HD_EXP_NOCONS
-    return s;
-#endif
     float4 r[2][8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) r[0][j] = buf[j * 64 + lane];
