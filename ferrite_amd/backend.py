@@ -70,7 +70,7 @@ EXPORTS = [
     "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_matmul_f32",
     "ferrite_swiglu_limited_f32", "ferrite_moe_route", "ferrite_moe_permute_scratch_bytes", "ferrite_moe_permute",
     "ferrite_mxfp4_dequant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes", "ferrite_moe_pack_weights",
-    "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
+    "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
     "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_timed", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
     "ferrite_graph_destroy",
 ]
@@ -99,6 +99,7 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_moe_pack_weights.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp]
     lib.ferrite_moe_packed_dequant.argtypes = [C.POINTER(MoeShape), vp, i32, i32, vp, vp]
     lib.ferrite_moe_layer_workspace_bytes.restype = sz
+    lib.ferrite_moe_layer_unit_rows.argtypes = [C.POINTER(MoeShape), i32, i32]
     lib.ferrite_moe_layer_workspace_bytes.argtypes = [C.POINTER(MoeShape), i32, i32]
     lib.ferrite_moe_layer_workspace_init.argtypes = [C.POINTER(MoeShape), i32, i32, vp, sz, vp]
     lib.ferrite_moe_layer_workspace_view.argtypes = [C.POINTER(MoeShape), i32, i32, vp, C.POINTER(WorkspaceView)]
@@ -409,6 +410,10 @@ class HipBackend:
             self._leave()
             layer._ws[key] = ws
         return layer._ws[key]
+
+    def unit_rows(self, layer: MoeLayer, n: int, mode: int = MODE_MFMA_FP8) -> int:
+        """Token tile of the expert GEMMs for such a call: 16 (streaming kernels) or 128 (LDS-tiled kernels)."""
+        return int(self.lib.ferrite_moe_layer_unit_rows(C.byref(layer.shape), n, mode))
 
     def moe_layer_dev_mxfp4(self, layer: MoeLayer, x: torch.Tensor, out: torch.Tensor, mode: int = MODE_MFMA_FP8,
                             workspace: Optional[torch.Tensor] = None, stage_events=None):

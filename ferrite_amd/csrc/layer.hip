@@ -109,6 +109,11 @@ extern "C" const char* ferrite_kernel_build_id(void) { return FERRITE_BUILD_ID; 
 extern "C" unsigned ferrite_kernel_abi_version(void) { return FERRITE_ABI_VERSION; }
 extern "C" const char* ferrite_hip_last_error(void) { return g_last_error; }
 
+extern "C" int ferrite_moe_layer_unit_rows(const ferrite_moe_shape* shape, int n, int mode) {
+    if (check_shape(shape, n, mode)) return 0;
+    return carve(*shape, n, mode).unit_cap;
+}
+
 extern "C" size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode) {
     if (check_shape(shape, n, mode)) return 0;
     return carve(*shape, n, mode).total;

@@ -142,6 +142,12 @@ typedef struct ferrite_moe_workspace_view {
 } ferrite_moe_workspace_view;
 
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
+/* Rows per unit (the token tile of the expert GEMMs) a layer call with these arguments uses: 16 = weights streamed
+ * once per unit (decode-sized batches), 128 = both operands tiled through LDS (prefill-sized batches); 0 for an
+ * unsupported shape.  The choice is a pure function of (shape, n, mode) and of the environment variable
+ * FERRITE_HIP_UNIT_ROWS (16 or 128 forces it, read at every call), like the workspace layout that depends on it.
+ * No counterpart in the reference, whose grouped GEMM has one tile shape (dsv41_moe.cu); informational. */
+int ferrite_moe_layer_unit_rows(const ferrite_moe_shape* shape, int n, int mode);
 /* Must run once on a freshly allocated workspace before its first layer call (it clears the arrival counters
  * the fused routing kernel keeps there; the kernel leaves them cleared, so replays need no further call).
  * Workspaces are owned by the caller like every other buffer (DevBuf pool, cuda.rs:558-744). */
