@@ -28,8 +28,9 @@ MFMA_PEAK_FP4_TFLOPS = 10100.0 # dense MXFP4 x MXFP4
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
 # counters' reading for a 1 GiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw values
-# are in profiles/c1_decode32_hbm_counters.md.  Counters cannot be read inside this script.
-MEASURED_TRAFFIC = {("c1", "gate_up_mfma_kernel"): 770.6e6}
+# are in profiles/c1_decode32_hbm_counters.md and profiles/c2_prefill4096_hbm_counters.md.  Counters cannot be read
+# inside this script.
+MEASURED_TRAFFIC = {("c1", "gate_up_mfma_kernel"): 770.5e6, ("c2", "gate_up_prefill_kernel"): 1832.8e6}
 
 WORKLOADS = {
     "c0": "c0: tiny parity layer, 8 tokens, H256 E16 top4 (4 groups/2) I128, MXFP4 weights, f32 activations",
@@ -208,6 +209,8 @@ def main():
                     "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_FP8_TFLOPS, 4),
                     "traffic": None, "algorithmic_flops_per_launch": gu_flops, "avg_launch_us": round(gu_us, 2),
                     "frac_of_fp4_peak": round(tf / MFMA_PEAK_FP4_TFLOPS, 4)}
+        if not args.tokens:
+            roofline["traffic"] = MEASURED_TRAFFIC.get((args.config, "gate_up_prefill_kernel"))
 
     cpu = None
     if not args.no_cpu_baseline:
