@@ -458,6 +458,9 @@ class HipBackend:
             return ws[off:off + count * size].view(dtype)
 
         E, k = cfg.n_experts, cfg.topk
+        y_bf16 = (mode == MODE_MFMA_FP8 and self.unit_rows(layer, n, mode) == 128
+                  and os.environ.get("FERRITE_HIP_Y_F32") != "1")
+        y_dtype = torch.bfloat16 if y_bf16 else torch.float32
         return dict(logits=view(v.logits, n * E, torch.float32).view(n, E),
                     probs=view(v.probs, n * k, torch.float32).view(n, k),
                     ids_f32=view(v.ids_f32, n * k, torch.float32).view(n, k),
@@ -465,7 +468,7 @@ class HipBackend:
                     counts=view(v.counts, E, torch.int32), starts=view(v.starts, E + 1, torch.int32),
                     perm_map=view(v.perm_map, n * k, torch.int32), gather_src=view(v.gather_src, n * k, torch.int32),
                     active=view(v.active, E, torch.int32), n_active=view(v.n_active, 1, torch.int32),
-                    y=view(v.y, rows * cfg.hidden, torch.float32).view(rows, cfg.hidden))
+                    y=view(v.y, rows * cfg.hidden, y_dtype).view(rows, cfg.hidden))
 
     # ---- GraphCapable (graph.rs:48-64; device semantics of cuda.rs:3043-3092) ----
     def begin_capture(self):

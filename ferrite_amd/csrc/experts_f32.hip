@@ -123,8 +123,19 @@ __global__ __launch_bounds__(256) void down_f32_kernel(ferrite_moe_shape s, ferr
 
 // out[t] = sum_j (ascending) probs[t,j] * y[perm_map[t*k+j]]  then  + y[n*k + t]   (exec/lib.rs:1154-1164:
 // a rounded product and a rounded add per slot, the shared expert last)
-template <typename OT>
-__global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ y, const float* __restrict__ probs,
+// four consecutive y values of a row: f32, or bf16 widened (exact)
+template <typename YT>
+__device__ __forceinline__ float4 load_y4(const YT* p) {
+    if constexpr (sizeof(YT) == 4) {
+        return *reinterpret_cast<const float4*>(p);
+    } else {
+        const uint2 q = *reinterpret_cast<const uint2*>(p);
+        return make_float4(u2f(q.x << 16), u2f(q.x & 0xffff0000u), u2f(q.y << 16), u2f(q.y & 0xffff0000u));
+    }
+}
+
+template <typename OT, typename YT>
+__global__ __launch_bounds__(256) void combine_kernel(const YT* __restrict__ y, const float* __restrict__ probs,
                                                       const int32_t* __restrict__ perm_map, int n, int topk,
                                                       int H, int has_shared, OT* __restrict__ out) {
     const int t = blockIdx.y;
@@ -135,12 +146,12 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* __restrict__ 
         int g = perm_map[(size_t)t * topk + j];
         if (g < 0 || g >= n * topk) continue;   // tables of an uninitialised workspace must not cause a fault
         float p = probs[(size_t)t * topk + j];
-        float4 v = *reinterpret_cast<const float4*>(y + (size_t)g * H + h);
+        float4 v = load_y4(y + (size_t)g * H + h);
         o.x = fadd(o.x, fmul(p, v.x)); o.y = fadd(o.y, fmul(p, v.y));
         o.z = fadd(o.z, fmul(p, v.z)); o.w = fadd(o.w, fmul(p, v.w));
     }
     if (has_shared) {
-        float4 v = *reinterpret_cast<const float4*>(y + ((size_t)n * topk + t) * H + h);
+        float4 v = load_y4(y + ((size_t)n * topk + t) * H + h);
         o.x = fadd(o.x, v.x); o.y = fadd(o.y, v.y); o.z = fadd(o.z, v.z); o.w = fadd(o.w, v.w);
     }
     if constexpr (sizeof(OT) == 4) {
@@ -177,15 +188,19 @@ int launch_down_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, co
     return check_launch("down_f32");
 }
 
-int launch_combine(const float* y, const float* probs, const int32_t* perm_map, int n, int topk, int hidden,
-                   int has_shared, void* out, int out_dtype, hipStream_t st) {
+int launch_combine(const void* y, int y_dtype, const float* probs, const int32_t* perm_map, int n, int topk,
+                   int hidden, int has_shared, void* out, int out_dtype, hipStream_t st) {
     dim3 grid((hidden / 4 + 255) / 256, n);
-    if (out_dtype == FERRITE_DT_F32)
-        combine_kernel<float><<<grid, 256, 0, st>>>(y, probs, perm_map, n, topk, hidden, has_shared, (float*)out);
-    else if (out_dtype == FERRITE_DT_BF16)
-        combine_kernel<uint16_t><<<grid, 256, 0, st>>>(y, probs, perm_map, n, topk, hidden, has_shared, (uint16_t*)out);
+    const bool of32 = out_dtype == FERRITE_DT_F32, yf32 = y_dtype == FERRITE_DT_F32;
+    if ((!of32 && out_dtype != FERRITE_DT_BF16) || (!yf32 && y_dtype != FERRITE_DT_BF16)) return FERRITE_ERR_INVALID_ARG;
+    if (of32 && yf32)
+        combine_kernel<float, float><<<grid, 256, 0, st>>>((const float*)y, probs, perm_map, n, topk, hidden, has_shared, (float*)out);
+    else if (of32)
+        combine_kernel<float, uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)y, probs, perm_map, n, topk, hidden, has_shared, (float*)out);
+    else if (yf32)
+        combine_kernel<uint16_t, float><<<grid, 256, 0, st>>>((const float*)y, probs, perm_map, n, topk, hidden, has_shared, (uint16_t*)out);
     else
-        return FERRITE_ERR_INVALID_ARG;
+        combine_kernel<uint16_t, uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)y, probs, perm_map, n, topk, hidden, has_shared, (uint16_t*)out);
     return check_launch("combine");
 }
 

@@ -581,8 +581,16 @@ __global__ __launch_bounds__(256, 2) void gate_up_prefill_kernel(MfmaArgs a, int
     }
 }
 
+// f32 -> bf16, round to nearest even (NaN stays NaN)
+__device__ __forceinline__ uint32_t bf16_rne(float f) {
+    const uint32_t u = f2u(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+template <typename YT>
 __global__ __launch_bounds__(256, 2) void down_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
-                                                           const uint8_t* __restrict__ act_s, float* __restrict__ y) {
+                                                           const uint8_t* __restrict__ act_s, YT* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig;
     if (!pf_block_work(*a.n_units, groups, u, ig)) return;
@@ -610,11 +618,16 @@ __global__ __launch_bounds__(256, 2) void down_prefill_kernel(MfmaArgs a, int gr
         for (int tt = 0; tt < 4; ++tt) {
             const int col = (c.wt * 4 + tt) * 16 + cc;
             if (col < nrows) {
-                float* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
+                YT* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    *reinterpret_cast<float4*>(dst + t * 16) =
-                        make_float4(acc[ii][t][tt][0], acc[ii][t][tt][1], acc[ii][t][tt][2], acc[ii][t][tt][3]);
+                for (int t = 0; t < 4; ++t) {
+                    const v4f r = acc[ii][t][tt];
+                    if constexpr (sizeof(YT) == 4)
+                        *reinterpret_cast<float4*>(dst + t * 16) = make_float4(r[0], r[1], r[2], r[3]);
+                    else
+                        *reinterpret_cast<uint2*>(dst + t * 16) =
+                            make_uint2(bf16_rne(r[0]) | (bf16_rne(r[1]) << 16), bf16_rne(r[2]) | (bf16_rne(r[3]) << 16));
+                }
             }
         }
     }
@@ -669,15 +682,15 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
 }
 
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
-                     int n, const UnitTables& units, float* y, hipStream_t st) {
+                     int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
     MfmaArgs a = make_args(s, packed, n, units, true);
     if (units.unit_rows_cap == PF_ROWS) {
-        static size_t raised_pf = 0;
-        int rc = set_lds_limit(down_prefill_kernel, PF_LDS_BYTES, &raised_pf);
-        if (rc) return rc;
         const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-        down_prefill_kernel<<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, y);
+        if (y_dtype == FERRITE_DT_BF16)
+            down_prefill_kernel<uint16_t><<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<uint16_t*>(y));
+        else
+            down_prefill_kernel<float><<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
         return check_launch("down_prefill");
     }
     if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
@@ -687,7 +700,8 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ui
     if (rc) return rc;
     const int items = s.hidden / 64;
     dim3 grid((items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW), units.max_units);
-    down_mfma_kernel<DN_WAVES, DN_IPW><<<grid, DN_WAVES * 64, lds, st>>>(a, act_q, act_s, y);
+    if (y_dtype != FERRITE_DT_F32) return FERRITE_ERR_INVALID_ARG;
+    down_mfma_kernel<DN_WAVES, DN_IPW><<<grid, DN_WAVES * 64, lds, st>>>(a, act_q, act_s, static_cast<float*>(y));
     return check_launch("down_mfma");
 }
 

@@ -37,6 +37,9 @@ inline int max_units_for(int n, int topk, int n_experts, int has_shared, int uni
 // sees enough rows to fill them, 16-row units (weights streamed once per unit) below that.  The environment
 // variable FERRITE_HIP_UNIT_ROWS (16 or 128) overrides the choice; it is read at every call.
 int unit_rows_for(int n, int topk, int n_experts);
+// Element type of the expert outputs `y` in the workspace: bf16 for 128-row units (prefill-sized batches, where the
+// y round trip through HBM is a tenth of the layer), f32 otherwise.  FERRITE_HIP_Y_F32=1 forces f32 (tests).
+int y_dtype_for(int unit_rows);
 
 // Kernels that need more than 64 KiB of dynamic LDS must have the limit raised once (a function attribute,
 // not a stream operation).  `raised` remembers the largest value already set for that kernel.
@@ -73,8 +76,8 @@ int launch_gate_up_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w,
                        const int32_t* ids, const int32_t* gather_src, float* act, hipStream_t st);
 int launch_down_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, const float* act, int n,
                     const int32_t* ids, const int32_t* gather_src, float* y, hipStream_t st);
-int launch_combine(const float* y, const float* probs, const int32_t* perm_map, int n, int topk, int hidden,
-                   int has_shared, void* out, int out_dtype, hipStream_t st);
+int launch_combine(const void* y, int y_dtype, const float* probs, const int32_t* perm_map, int n, int topk,
+                   int hidden, int has_shared, void* out, int out_dtype, hipStream_t st);
 
 // experts_mfma.hip
 struct PackedLayout {
@@ -90,7 +93,7 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
                         int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
                         hipStream_t st);
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
-                     int n, const UnitTables& units, float* y, hipStream_t st);
+                     int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st);
 
 // formats.hip
 int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, int operand_order,

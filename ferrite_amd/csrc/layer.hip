@@ -43,6 +43,12 @@ int unit_rows_for(int n, int topk, int n_experts) {
     return (long)n * topk >= 48L * n_experts ? 128 : 16;
 }
 
+int y_dtype_for(int unit_rows) {
+    if (unit_rows != 128) return FERRITE_DT_F32;
+    const char* v = getenv("FERRITE_HIP_Y_F32");
+    return (v && !strcmp(v, "1")) ? FERRITE_DT_F32 : FERRITE_DT_BF16;
+}
+
 static size_t bump(size_t& off, size_t bytes) {
     size_t at = off;
     off = (off + bytes + 255) / 256 * 256;
@@ -191,7 +197,8 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     int32_t* ids = reinterpret_cast<int32_t*>(b + w.ids);
     int32_t* perm_map = reinterpret_cast<int32_t*>(b + w.perm_map);
     int32_t* gather_src = reinterpret_cast<int32_t*>(b + w.gather_src);
-    float* y = reinterpret_cast<float*>(b + w.y);
+    void* y = b + w.y;
+    const int y_dtype = mode == FERRITE_MODE_MFMA_FP8 ? y_dtype_for(w.unit_cap) : FERRITE_DT_F32;
 
     UnitTables units{reinterpret_cast<int32_t*>(b + w.unit_expert), reinterpret_cast<int32_t*>(b + w.unit_row0),
                      reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.n_units), w.unit_cap,
@@ -246,17 +253,17 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         float* act = reinterpret_cast<float*>(b + w.act);
         if ((rc = launch_gate_up_f32(s, *wts, static_cast<const float*>(x), n, ids, gather_src, act, st))) return rc;
         if ((rc = mark(ev, 5, st))) return rc;
-        if ((rc = launch_down_f32(s, *wts, act, n, ids, gather_src, y, st))) return rc;
+        if ((rc = launch_down_f32(s, *wts, act, n, ids, gather_src, static_cast<float*>(y), st))) return rc;
     } else {
         uint8_t* act_q = reinterpret_cast<uint8_t*>(b + w.act);
         uint8_t* act_s = reinterpret_cast<uint8_t*>(b + w.act_s);
         if ((rc = launch_gate_up_mfma(s, packed, xq, xs, n, gather_src, units, act_q, act_s, st))) return rc;
         if ((rc = mark(ev, 5, st))) return rc;
-        if ((rc = launch_down_mfma(s, packed, act_q, act_s, n, units, y, st))) return rc;
+        if ((rc = launch_down_mfma(s, packed, act_q, act_s, n, units, y, y_dtype, st))) return rc;
     }
     if ((rc = mark(ev, 6, st))) return rc;
     // 6. weighted combine in slot order + shared expert (exec/lib.rs:1154-1164)
-    if ((rc = launch_combine(y, probs, perm_map, n, s.topk, s.hidden, has_shared, out, out_dtype, st))) return rc;
+    if ((rc = launch_combine(y, y_dtype, probs, perm_map, n, s.topk, s.hidden, has_shared, out, out_dtype, st))) return rc;
     return mark(ev, 7, st);
 }
 

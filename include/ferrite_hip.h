@@ -138,7 +138,9 @@ typedef struct ferrite_moe_workspace_view {
     int32_t* gather_src; /* [n*topk] */
     int32_t* active;     /* [E] */
     int32_t* n_active;   /* [1] */
-    float* y;            /* [(n*topk + n), H] expert outputs in grouped order, then the shared expert's rows */
+    float* y;            /* [(n*topk + n), H] expert outputs in grouped order, then the shared expert's rows; f32,
+                          * except bf16 (same shape, half the bytes) when ferrite_moe_layer_unit_rows() is 128 and
+                          * FERRITE_HIP_Y_F32=1 is not set in the environment */
 } ferrite_moe_workspace_view;
 
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
