@@ -387,7 +387,11 @@ __device__ __forceinline__ void pf_fill(const PfCtx& c, u4v* stage, int kt) {
 }
 
 // All loads into LDS issued by this wave have landed (vmcnt 0; expcnt and lgkmcnt left alone).
+#ifdef PF_EXP_NOWAIT
+__device__ __forceinline__ void pf_wait_fill() {}
+#else
 __device__ __forceinline__ void pf_wait_fill() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+#endif
 
 // One k step: operands of the current stage into registers, then the next stage's loads are started (after the
 // operand reads in program order: the compiler cannot tell the two stages apart and would otherwise wait for the

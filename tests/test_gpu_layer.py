@@ -177,6 +177,57 @@ def test_layer_unfused_head_path(hip, oracle):
     assert max_abs_rel(out, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
 
 
+@pytest.mark.parametrize("n", [40, 700])
+def test_layer_all_tokens_on_the_same_experts(hip, oracle, n):
+    """Maximum skew: a bias of +50 on three experts of one group makes every token pick exactly those (the sigmoid
+    is at most 1), so three experts hold n rows each (full 16- / 128-row units plus a ragged tail) and thirteen hold
+    none."""
+    cfg = synth.MoeConfig(n, 256, 16, 3, 128, 128, 4, 2)
+    inp = synth.make_inputs(cfg, seed=21)
+    inp.router_bias[:] = 0.0
+    inp.router_bias[[4, 5, 7]] = 50.0
+    layer = hip.load_moe_layer(inp)
+    ref32 = oracle.moe_ffn_mxfp4(inp, n_threads=8)
+    assert set(np.unique(ref32["ids"]).astype(int)) == {4, 5, 7}
+    out, v = run_layer(hip, layer, inp.x, MODE_F32_CHECK)
+    check_routing(v, ref32, oracle, cfg)
+    assert v["counts"].max() == n and (v["counts"] > 0).sum() == 3
+    assert max_abs_rel(out, ref32["out"]) <= TOL_F32
+    out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    check_routing(v, ref32, oracle, cfg)
+    assert max_abs_rel(out, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
+
+
+def test_layer_error_paths(hip):
+    """Argument errors are reported by return code before anything is launched (cuda.rs:411-425 conventions)."""
+    from ferrite_amd.backend import Declined, FerriteError, InvalidArg, ShapeMismatch
+    cfg = synth.CONFIGS["c0"]
+    inp = synth.make_inputs(cfg, seed=0)
+    layer = hip.load_moe_layer(inp)
+    x = torch.from_numpy(inp.x).to(hip.device)
+    out = torch.empty_like(x)
+    with pytest.raises(ShapeMismatch):
+        hip.moe_layer_dev_mxfp4(layer, x[:, :128].contiguous(), out, MODE_MFMA_FP8)
+    with pytest.raises(InvalidArg):
+        hip.moe_layer_dev_mxfp4(layer, x, out[:4], MODE_MFMA_FP8)
+    with pytest.raises(FerriteError):          # the f32 check mode takes f32 activations only
+        hip.moe_layer_dev_mxfp4(layer, x.to(torch.bfloat16), out, MODE_F32_CHECK)
+    small = torch.empty(1024, dtype=torch.uint8, device=hip.device)
+    with pytest.raises(FerriteError):          # FERRITE_ERR_WORKSPACE
+        hip.moe_layer_dev_mxfp4(layer, x, out, MODE_MFMA_FP8, workspace=small)
+    # hidden not a multiple of 128: the MFMA mode declines at packing time, the f32 mode still runs
+    odd = synth.make_inputs(synth.MoeConfig(4, 64, 8, 2, 64, 64, 1, 1), seed=1)
+    with pytest.raises((Declined, InvalidArg)):
+        hip.load_moe_layer(odd)
+    ly = hip.load_moe_layer(odd, pack=False)
+    xo = torch.from_numpy(odd.x).to(hip.device)
+    oo = torch.empty_like(xo)
+    hip.moe_layer_dev_mxfp4(ly, xo, oo, MODE_F32_CHECK)
+    with pytest.raises(FerriteError):
+        hip.moe_layer_dev_mxfp4(ly, xo, oo, MODE_MFMA_FP8)
+    hip.sync()
+
+
 def test_layer_repeated_calls_same_workspace(hip, oracle):
     """The fused routing kernel keeps arrival counters in the workspace and must leave them cleared."""
     inp = synth.make_inputs(synth.CONFIGS["c0"].with_tokens(40), seed=3)
