@@ -387,11 +387,7 @@ __device__ __forceinline__ void pf_fill(const PfCtx& c, u4v* stage, int kt) {
 }
 
 // All loads into LDS issued by this wave have landed (vmcnt 0; expcnt and lgkmcnt left alone).
-#ifdef PF_EXP_NOWAIT
-__device__ __forceinline__ void pf_wait_fill() {}
-#else
 __device__ __forceinline__ void pf_wait_fill() { __builtin_amdgcn_s_waitcnt(0x0F70); }
-#endif
 
 // One k step: operands of the current stage into registers, then the next stage's loads are started (after the
 // operand reads in program order: the compiler cannot tell the two stages apart and would otherwise wait for the
@@ -502,13 +498,14 @@ __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const
     c.a_src = reinterpret_cast<const u4v*>(cbase) + (size_t)min(item0 + c.wave, items - 1) * KT * 256 + c.lane;
     // Activation stage layout: the four lanes of a quad fetch 64 consecutive bytes of one row (what the texture
     // addresser coalesces), so row r's 16-byte chunk q of a half k step lands at slot 4r + q; the chunk a lane
-    // fetches is XORed with r/4 so that the operand read of 16 rows at a fixed chunk is spread over all banks.
+    // fetches is XORed with (r/2)%4 so that any eight consecutive lanes of the operand read (rows r..r+7 at a fixed
+    // chunk) touch eight different 16-byte bank groups (counters: no LDS bank conflicts; XOR with r/4 had them).
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int col = (c.wave * 2 + i) * 16 + (c.lane >> 2);
-        c.b_src[i] = row_q(col < nrows ? col : 0) + ((c.lane & 3) ^ (c.lane >> 4)) * 16;
+        c.b_src[i] = row_q(col < nrows ? col : 0) + ((c.lane & 3) ^ ((c.lane >> 3) & 3)) * 16;
     }
-    c.bslot = 4 * cc + (g ^ (cc >> 2));
+    c.bslot = 4 * cc + (g ^ ((cc >> 1) & 3));
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
         const int item = min(item0 + c.wi * 2 + ii, items - 1);
