@@ -65,7 +65,7 @@ bool head_supported(int n, int H, int E);
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
                     int n, float* logits, float* probs, float* ids_f32, int32_t* ids, uint8_t* xq, uint8_t* xs,
                     int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
-                    int32_t* active, int32_t* n_active, const UnitTables* units, hipStream_t st);
+                    int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, hipStream_t st);
 int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
                         hipStream_t st);
 int launch_router_transpose(const float* w, int E, int H, float* dst, hipStream_t st);

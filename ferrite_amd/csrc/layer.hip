@@ -210,14 +210,23 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     if (fused_head) {
         // 1-3 (+ activation quantisation) as one launch
         PackedLayout L = packed_layout(s);
+        const int fuse_perm = n <= 64;
         if ((rc = launch_moe_head(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), wts->router_bias, s,
                                   n, logits, probs, ids_f32, ids, xq, xs, reinterpret_cast<int32_t*>(b + w.counters),
                                   reinterpret_cast<int32_t*>(b + w.counts), reinterpret_cast<int32_t*>(b + w.starts),
                                   perm_map, gather_src, reinterpret_cast<int32_t*>(b + w.active),
-                                  reinterpret_cast<int32_t*>(b + w.n_active), &units, st)))
+                                  reinterpret_cast<int32_t*>(b + w.n_active), &units, fuse_perm, st)))
             return rc;
-        for (int i = 1; i <= 4; ++i)
-            if ((rc = mark(ev, i, st))) return rc;
+        if ((rc = mark(ev, 1, st))) return rc;
+        if ((rc = mark(ev, 2, st))) return rc;
+        if (!fuse_perm &&
+            (rc = launch_permute(ids, n, s.topk, s.n_experts, reinterpret_cast<int32_t*>(b + w.counts),
+                                 reinterpret_cast<int32_t*>(b + w.starts), perm_map, gather_src,
+                                 reinterpret_cast<int32_t*>(b + w.active), reinterpret_cast<int32_t*>(b + w.n_active),
+                                 b + w.perm_scratch, w.perm_scratch_bytes, &units, has_shared, st)))
+            return rc;
+        if ((rc = mark(ev, 3, st))) return rc;
+        if ((rc = mark(ev, 4, st))) return rc;
     } else {
     // 1. router logits: the reference's sequential-k f32 chain (exec/lib.rs:1107)
     if (packed != nullptr && s.hidden % 128 == 0) {

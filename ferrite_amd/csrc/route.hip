@@ -519,25 +519,25 @@ __global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const 
 // ------------------------------------------------------------------------------------------------
 // The head of the layer as ONE launch (decode-sized batches), or the router GEMM alone (kFused = false).
 // Workgroups have eight waves.
-//   blocks (eb, t), eb < eblocks : router logits of token t for experts [64 eb, 64 eb + 64): the reference's
+//   blocks (eb, tg), eb < eblocks: router logits of the tokens of group tg for experts [64 eb, 64 eb + 64): the reference's
 //                                  sequential chain, one lane of wave 0 per expert.  A lone wave issues one
 //                                  instruction every four cycles, loads and address arithmetic included, so the
 //                                  chain wave is left with nothing but the adds: six producer waves fetch the router
 //                                  weight (k-blocked transpose [H/4][Epad][4], four chunks ahead), multiply it
 //                                  with x[t] (the products are order-independent and each rounded once, as in
-//                                  the reference) and hand the products over through a two-buffer LDS ring of
-//                                  32-group chunks; wave 0 reads them back and adds them in k order
+//                                  the reference) and hand the products over through a two-buffer LDS ring;
+//                                  wave 0 reads them back and adds them in k order.  When one token per
+//                                  block would need more than one round of blocks, a block takes two tokens
+//                                  (two interleaved chains in wave 0, the weights fetched once for both)
 //   blocks (eblocks, t)          : e4m3-per-32 quantisation of x[t] (off the critical path)
 //   last logits block of a token : its wave 0 routes the token (arrival counter per token)
-//   last routed token            : builds the permutation and unit tables, then clears the counters so the
-//                                  next launch (or graph replay) starts clean
+//   last routed token            : builds the permutation and unit tables (up to 64 tokens; above that one wave
+//                                  is too slow for it and a separate launch follows), then clears the counters
+//                                  so the next launch (or graph replay) starts clean
 // counters[0] = routed tokens, counters[1 + t] = logits blocks of token t that have arrived; all zero on entry.
 // ------------------------------------------------------------------------------------------------
 constexpr int HEAD_MAX_N = 256;
-constexpr int HD_CH = 32;                              // groups of four k per chunk
 constexpr int HD_NP = 6;                               // producer waves
-constexpr int HD_PW = (HD_CH + HD_NP - 1) / HD_NP;     // groups per producer wave and chunk (6 or 5)
-constexpr size_t HD_RING_BYTES = 2 * (size_t)HD_CH * 1024;
 
 struct HeadArgs {
     const void* x;
@@ -549,76 +549,99 @@ struct HeadArgs {
     int32_t* ids;
     uint8_t *xq, *xs;     // may be NULL: no quantisation blocks are launched then
     int32_t* counters;    // [1 + n]
+    int fuse_perm;        // the last routed token also builds the permutation (small n); else a separate launch does
     PermArgs perm;
 };
 
-struct HeadSet {
-    float4 w[HD_PW];
+// T = tokens per block (1, or 2 when one token per block would need more than one round of blocks on the chip).
+template <int T>
+struct HeadCfg {
+    static constexpr int CH = 32 / T;                        // groups of four k per chunk
+    static constexpr int PW = (CH + HD_NP - 1) / HD_NP;      // groups per producer wave and chunk
+    static constexpr size_t RING_BYTES = 2 * (size_t)CH * T * 1024;   // 64 KiB
 };
 
-// Producer P (0..HD_NP-1) owns groups P, P+HD_NP, ... of every chunk.  Chunks past the end re-read the last one (never
-// consumed), which keeps every load unconditional.
-template <int P>
-__device__ __forceinline__ void head_pload(HeadSet& st, const float4* __restrict__ wp, int Epad, int c, int nch) {
-    const float4* base = wp + (size_t)min(c, nch - 1) * HD_CH * Epad;
+template <int T>
+struct HeadSet {
+    float4 w[HeadCfg<T>::PW];
+};
+
+// Producer P (0..HD_NP-1) owns groups P, P+HD_NP, ... of every chunk.  Chunks past the end re-read the last one
+// (never consumed), which keeps every load unconditional.
+template <int T, int P>
+__device__ __forceinline__ void head_pload(HeadSet<T>& st, const float4* __restrict__ wp, int Epad, int c, int nch) {
+    constexpr int CH = HeadCfg<T>::CH;
+    const float4* base = wp + (size_t)min(c, nch - 1) * CH * Epad;
 #pragma unroll
-    for (int i = 0; i < HD_PW; ++i)
-        if (P + HD_NP * i < HD_CH) st.w[i] = base[(size_t)(P + HD_NP * i) * Epad];
+    for (int i = 0; i < HeadCfg<T>::PW; ++i)
+        if (P + HD_NP * i < CH) st.w[i] = base[(size_t)(P + HD_NP * i) * Epad];
 }
 
-template <int P>
-__device__ __forceinline__ void head_pmul(const HeadSet& st, const float4* xc, float4* buf, int lane) {
+// products of the chunk's group j for token ti go to slot (j*T + ti)*64 + lane of the ring buffer
+template <int T, int P>
+__device__ __forceinline__ void head_pmul(const HeadSet<T>& st, const float4* xl, int nk4, int c, float4* buf, int lane) {
+    constexpr int CH = HeadCfg<T>::CH;
 #pragma unroll
-    for (int i = 0; i < HD_PW; ++i) {
+    for (int i = 0; i < HeadCfg<T>::PW; ++i) {
         const int j = P + HD_NP * i;
-        if (j < HD_CH) {
-            const float4 xv = xc[j], wv = st.w[i];
-            buf[j * 64 + lane] = make_float4(fmul(xv.x, wv.x), fmul(xv.y, wv.y), fmul(xv.z, wv.z), fmul(xv.w, wv.w));
+        if (j < CH) {
+            const float4 wv = st.w[i];
+#pragma unroll
+            for (int ti = 0; ti < T; ++ti) {
+                const float4 xv = xl[ti * nk4 + c * CH + j];
+                buf[(j * T + ti) * 64 + lane] =
+                    make_float4(fmul(xv.x, wv.x), fmul(xv.y, wv.y), fmul(xv.z, wv.z), fmul(xv.w, wv.w));
+            }
         }
     }
 }
 
 // Products of chunk c+1 are made while the chain consumes chunk c; register set c%4 holds the weights of chunk c
 // and is reloaded for chunk c+4 as soon as it has been used.
-template <int P>
-__device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int Epad, int nch, const float4* xl,
+template <int T, int P>
+__device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int Epad, int nk4, const float4* xl,
                                               float4* ring, int lane) {
+    constexpr int CH = HeadCfg<T>::CH;
+    const int nch = nk4 / CH;
     float4* b0 = ring;
-    float4* b1 = ring + HD_CH * 64;
-    HeadSet s0, s1, s2, s3;
-    head_pload<P>(s0, wp, Epad, 0, nch);
-    head_pload<P>(s1, wp, Epad, 1, nch);
-    head_pload<P>(s2, wp, Epad, 2, nch);
-    head_pload<P>(s3, wp, Epad, 3, nch);
-    __syncthreads();   // x[t] is in LDS
-    head_pmul<P>(s0, xl, b0, lane);
-    head_pload<P>(s0, wp, Epad, 4, nch);
+    float4* b1 = ring + CH * T * 64;
+    HeadSet<T> s0, s1, s2, s3;
+    head_pload<T, P>(s0, wp, Epad, 0, nch);
+    head_pload<T, P>(s1, wp, Epad, 1, nch);
+    head_pload<T, P>(s2, wp, Epad, 2, nch);
+    head_pload<T, P>(s3, wp, Epad, 3, nch);
+    __syncthreads();   // x is in LDS
+    head_pmul<T, P>(s0, xl, nk4, 0, b0, lane);
+    head_pload<T, P>(s0, wp, Epad, 4, nch);
     __syncthreads();
     for (int c = 0; c < nch; c += 4) {
-        head_pmul<P>(s1, xl + min(c + 1, nch - 1) * HD_CH, b1, lane);
-        head_pload<P>(s1, wp, Epad, c + 5, nch);
+        head_pmul<T, P>(s1, xl, nk4, min(c + 1, nch - 1), b1, lane);
+        head_pload<T, P>(s1, wp, Epad, c + 5, nch);
         __syncthreads();
-        head_pmul<P>(s2, xl + min(c + 2, nch - 1) * HD_CH, b0, lane);
-        head_pload<P>(s2, wp, Epad, c + 6, nch);
+        head_pmul<T, P>(s2, xl, nk4, min(c + 2, nch - 1), b0, lane);
+        head_pload<T, P>(s2, wp, Epad, c + 6, nch);
         __syncthreads();
-        head_pmul<P>(s3, xl + min(c + 3, nch - 1) * HD_CH, b1, lane);
-        head_pload<P>(s3, wp, Epad, c + 7, nch);
+        head_pmul<T, P>(s3, xl, nk4, min(c + 3, nch - 1), b1, lane);
+        head_pload<T, P>(s3, wp, Epad, c + 7, nch);
         __syncthreads();
-        head_pmul<P>(s0, xl + min(c + 4, nch - 1) * HD_CH, b0, lane);
-        head_pload<P>(s0, wp, Epad, c + 8, nch);
+        head_pmul<T, P>(s0, xl, nk4, min(c + 4, nch - 1), b0, lane);
+        head_pload<T, P>(s0, wp, Epad, c + 8, nch);
         __syncthreads();
     }
 }
 
-// The chain over one chunk of products: batches of eight LDS reads, one wait per batch (0xC87F: lgkmcnt <= 8, i.e.
-// everything but the batch just issued; 0xC07F: lgkmcnt 0), 32 dependent adds per batch.
-__device__ __forceinline__ float head_consume(float s, const float4* buf, int lane) {
+// The chains over one chunk of products: batches of eight LDS reads (8/T groups of four k for each of the T
+// tokens), one wait per batch (0xC87F: lgkmcnt <= 8, i.e. everything but the batch just issued; 0xC07F: lgkmcnt 0),
+// 32 adds per batch, dependent within a token's chain.
+template <int T>
+__device__ __forceinline__ void head_consume(float (&s)[T], const float4* buf, int lane) {
+    constexpr int NB = HeadCfg<T>::CH * T / 8;   // batches per chunk (4)
     float4 r[2][8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) r[0][j] = buf[j * 64 + lane];
 #pragma unroll
-    for (int g = 0; g < HD_CH / 8; ++g) {
-        if (g + 1 < HD_CH / 8) {
+    for (int g = 0; g < NB; ++g) {
+        if (g + 1 < NB) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) r[(g + 1) & 1][j] = buf[((g + 1) * 8 + j) * 64 + lane];
             __builtin_amdgcn_sched_barrier(0);
@@ -628,108 +651,128 @@ __device__ __forceinline__ float head_consume(float s, const float4* buf, int la
             __builtin_amdgcn_s_waitcnt(0xC07F);
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < 8; ++j) {   // slot order is (group, token): j % T is the token
             const float4 p = r[g & 1][j];
-            s = fadd(s, p.x);
-            s = fadd(s, p.y);
-            s = fadd(s, p.z);
-            s = fadd(s, p.w);
+            float a = s[j % T];
+            a = fadd(a, p.x);
+            a = fadd(a, p.y);
+            a = fadd(a, p.z);
+            a = fadd(a, p.w);
+            s[j % T] = a;
         }
         __builtin_amdgcn_sched_barrier(0);
     }
-    return s;
 }
 
 // Barriers pair one to one with head_producer's.
-__device__ __forceinline__ float head_consumer(int nch, const float4* ring, int lane) {
+template <int T>
+__device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const float4* ring, int lane) {
+    constexpr int CH = HeadCfg<T>::CH;
+    const int nch = nk4 / CH;
     const float4* b0 = ring;
-    const float4* b1 = ring + HD_CH * 64;
-    float s = 0.0f;
+    const float4* b1 = ring + CH * T * 64;
     __syncthreads();
     __syncthreads();
     for (int c = 0; c < nch; c += 4) {
-        s = head_consume(s, b0, lane);
+        head_consume<T>(s, b0, lane);
         __syncthreads();
-        if (c + 1 < nch) s = head_consume(s, b1, lane);
+        if (c + 1 < nch) head_consume<T>(s, b1, lane);
         __syncthreads();
-        if (c + 2 < nch) s = head_consume(s, b0, lane);
+        if (c + 2 < nch) head_consume<T>(s, b0, lane);
         __syncthreads();
-        if (c + 3 < nch) s = head_consume(s, b1, lane);
+        if (c + 3 < nch) head_consume<T>(s, b1, lane);
         __syncthreads();
     }
-    return s;
 }
 
-template <typename XT, bool kFused>
+template <typename XT, bool kFused, int T>
 __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
     extern __shared__ __align__(16) unsigned char head_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int eb = blockIdx.x, t = blockIdx.y;
+    const int eb = blockIdx.x, t0 = blockIdx.y * T;
     const int eblocks = a.Epad >> 6;
     const int H = a.H;
-    const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
     if (eb == eblocks) {
-        for (int b = tid; b < H / 32; b += 512)
-            a.xs[(size_t)t * scale_pitch(H) + scale_pos(b)] =
-                (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
+        for (int ti = 0; ti < T; ++ti) {
+            const int t = t0 + ti;
+            if (t >= a.n) break;
+            const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
+            for (int b = tid; b < H / 32; b += 512)
+                a.xs[(size_t)t * scale_pitch(H) + scale_pos(b)] =
+                    (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
+        }
         return;
     }
     float4* ring = reinterpret_cast<float4*>(head_lds);
-    float4* xl = reinterpret_cast<float4*>(head_lds + HD_RING_BYTES);
-    const int nk4 = H / 4, nch = nk4 / HD_CH;   // H % 128 == 0
+    float4* xl = reinterpret_cast<float4*>(head_lds + HeadCfg<T>::RING_BYTES);   // [T][H/4]
+    const int nk4 = H / 4;   // a multiple of 32 (H % 128 == 0)
     const float4* wp = reinterpret_cast<const float4*>(a.wt) + (size_t)eb * 64 + lane;
-    for (int i = tid; i < nk4; i += 512) {
+    for (int i = tid; i < T * nk4; i += 512) {
+        const int ti = i / nk4, k4 = i - ti * nk4;
+        const XT* xrow = static_cast<const XT*>(a.x) + (size_t)min(t0 + ti, a.n - 1) * H;
         float4 v;
         if constexpr (sizeof(XT) == 4) {
-            v = reinterpret_cast<const float4*>(xrow)[i];
+            v = reinterpret_cast<const float4*>(xrow)[k4];
         } else {
-            uint2 q = reinterpret_cast<const uint2*>(xrow)[i];
+            uint2 q = reinterpret_cast<const uint2*>(xrow)[k4];
             v = make_float4(u2f(q.x << 16), u2f(q.x & 0xffff0000u), u2f(q.y << 16), u2f(q.y & 0xffff0000u));
         }
         xl[i] = v;
     }
     // wave 0 chains; wave 4 would share its SIMD (and its VALU issue slots) and leaves; the others produce
-    float s = 0.0f;
+    float s[T];
+#pragma unroll
+    for (int ti = 0; ti < T; ++ti) s[ti] = 0.0f;
     switch (wave) {
-        case 0: s = head_consumer(nch, ring, lane); break;
-        case 1: head_producer<0>(wp, a.Epad, nch, xl, ring, lane); break;
-        case 2: head_producer<1>(wp, a.Epad, nch, xl, ring, lane); break;
-        case 3: head_producer<2>(wp, a.Epad, nch, xl, ring, lane); break;
-        case 5: head_producer<3>(wp, a.Epad, nch, xl, ring, lane); break;
-        case 6: head_producer<4>(wp, a.Epad, nch, xl, ring, lane); break;
-        case 7: head_producer<5>(wp, a.Epad, nch, xl, ring, lane); break;
-        default: __syncthreads(); break;   // its share of x[t] is in LDS before it goes
+        case 0: head_consumer<T>(s, nk4, ring, lane); break;
+        case 1: head_producer<T, 0>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 2: head_producer<T, 1>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 3: head_producer<T, 2>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 5: head_producer<T, 3>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 6: head_producer<T, 4>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 7: head_producer<T, 5>(wp, a.Epad, nk4, xl, ring, lane); break;
+        default: __syncthreads(); break;   // its share of x is in LDS before it goes
     }
     if (wave != 0) return;   // from here on the block is wave 0 alone; LDS is free for the scratch below
     const int e = eb * 64 + lane;
-    if (e < a.E) a.logits[(size_t)t * a.E + e] = s;
-    if constexpr (!kFused) return;
-
-    // arrival: the stores above are made visible before the counter moves
-    __threadfence();
-    int last = 0;
-    if (lane == 0) last = atomicAdd(&a.counters[1 + t], 1) == eblocks - 1;
-    last = __shfl(last, 0, 64);
-    if (!last) return;
-    __threadfence();
-    wave_sync();
-    RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds);
-    route_wave<true>(a.logits + (size_t)t * a.E, a.bias, true, a.E, a.topk, a.n_group, a.topk_group, a.scaling, sc,
-                     a.probs + (size_t)t * a.topk, a.ids_f32 + (size_t)t * a.topk, a.ids + (size_t)t * a.topk);
-    __threadfence();
-    last = 0;
-    if (lane == 0) last = atomicAdd(&a.counters[0], 1) == a.n - 1;
-    last = __shfl(last, 0, 64);
-    if (!last) return;
-    __threadfence();
-    wave_sync();
-    permute_in_block<true, true>(a.perm, reinterpret_cast<unsigned long long*>(head_lds));
-    for (int i = lane; i < a.n + 1; i += 64) a.counters[i] = 0;
+#pragma unroll
+    for (int ti = 0; ti < T; ++ti) {
+        const int t = t0 + ti;
+        if (t >= a.n) break;
+        if (e < a.E) a.logits[(size_t)t * a.E + e] = s[ti];
+        if constexpr (kFused) {
+            // arrival: the stores above are made visible before the counter moves
+            __threadfence();
+            int last = 0;
+            if (lane == 0) last = atomicAdd(&a.counters[1 + t], 1) == eblocks - 1;
+            last = __shfl(last, 0, 64);
+            if (!last) continue;
+            __threadfence();
+            wave_sync();
+            RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds);
+            route_wave<true>(a.logits + (size_t)t * a.E, a.bias, true, a.E, a.topk, a.n_group, a.topk_group, a.scaling,
+                             sc, a.probs + (size_t)t * a.topk, a.ids_f32 + (size_t)t * a.topk,
+                             a.ids + (size_t)t * a.topk);
+            __threadfence();
+            last = 0;
+            if (lane == 0) last = atomicAdd(&a.counters[0], 1) == a.n - 1;
+            last = __shfl(last, 0, 64);
+            if (!last) continue;
+            __threadfence();
+            wave_sync();
+            if (a.fuse_perm) permute_in_block<true, true>(a.perm, reinterpret_cast<unsigned long long*>(head_lds));
+            for (int i = lane; i < a.n + 1; i += 64) a.counters[i] = 0;
+        }
+    }
 }
 
+// tokens per block: two when one per block would not fit the chip's 256 CUs in one round
+static int head_tokens_per_block(int n, int eblocks) { return (long)n * eblocks > 256 ? 2 : 1; }
+
 static size_t head_lds_bytes(int n, int H, int E, bool fused) {
-    size_t b = HD_RING_BYTES + (size_t)H * 4;
+    const int T = head_tokens_per_block(n, (E + 63) / 64);
+    size_t b = 64 * 1024 + (size_t)T * H * 4;
     if (fused) {
         if (b < sizeof(RouteScratch)) b = sizeof(RouteScratch);
         size_t p = perm_block_lds_bytes(n, E);
@@ -742,19 +785,26 @@ bool head_supported(int n, int H, int E) {
     return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, H, E, true) <= 160 * 1024;
 }
 
-template <typename XT, bool kFused>
-static int launch_head_t(const HeadArgs& a, dim3 grid, size_t lds, hipStream_t st) {
+template <typename XT, bool kFused, int T>
+static int launch_head_tt(const HeadArgs& a, int quant, size_t lds, hipStream_t st) {
     static size_t raised = 0;
-    int rc = set_lds_limit(moe_head_kernel<XT, kFused>, lds, &raised);
+    int rc = set_lds_limit(moe_head_kernel<XT, kFused, T>, lds, &raised);
     if (rc) return rc;
-    moe_head_kernel<XT, kFused><<<grid, 512, lds, st>>>(a);
+    dim3 grid(a.Epad / 64 + quant, (a.n + T - 1) / T);
+    moe_head_kernel<XT, kFused, T><<<grid, 512, lds, st>>>(a);
     return check_launch("moe_head");
+}
+
+template <typename XT, bool kFused>
+static int launch_head_t(const HeadArgs& a, int quant, size_t lds, hipStream_t st) {
+    if (head_tokens_per_block(a.n, a.Epad / 64) == 2) return launch_head_tt<XT, kFused, 2>(a, quant, lds, st);
+    return launch_head_tt<XT, kFused, 1>(a, quant, lds, st);
 }
 
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
                     int n, float* logits, float* probs, float* ids_f32, int32_t* ids, uint8_t* xq, uint8_t* xs,
                     int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
-                    int32_t* active, int32_t* n_active, const UnitTables* units, hipStream_t st) {
+                    int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, hipStream_t st) {
     if (!head_supported(n, s.hidden, s.n_experts)) return FERRITE_DECLINED;
     HeadArgs a{};
     a.x = x; a.wt = router_t; a.bias = bias;
@@ -762,6 +812,7 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
     a.n_group = (s.n_group > 1 && s.topk_group < s.n_group) ? s.n_group : 1;
     a.topk_group = s.topk_group; a.scaling = s.routed_scaling;
     a.logits = logits; a.probs = probs; a.ids_f32 = ids_f32; a.ids = ids; a.xq = xq; a.xs = xs; a.counters = counters;
+    a.fuse_perm = fuse_perm;
     PermArgs& p = a.perm;
     p.ids = ids; p.n = n; p.topk = s.topk; p.n_experts = s.n_experts;
     p.counts = counts; p.starts = starts; p.perm_map = perm_map; p.gather_src = gather_src;
@@ -770,10 +821,9 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
         p.unit_expert = units->unit_expert; p.unit_row0 = units->unit_row0; p.unit_rows = units->unit_rows;
         p.n_units = units->n_units; p.unit_cap = units->unit_rows_cap; p.max_units = units->max_units;
     }
-    dim3 grid(a.Epad / 64 + (xq ? 1 : 0), n);
     const size_t lds = head_lds_bytes(n, s.hidden, s.n_experts, true);
-    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, grid, lds, st);
-    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, true>(a, grid, lds, st);
+    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, xq ? 1 : 0, lds, st);
+    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, true>(a, xq ? 1 : 0, lds, st);
     return FERRITE_ERR_INVALID_ARG;
 }
 
@@ -918,10 +968,9 @@ int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n
     if (head_lds_bytes(n, H, E, false) > 160 * 1024) return FERRITE_DECLINED;
     HeadArgs a{};
     a.x = x; a.wt = router_t; a.n = n; a.H = H; a.E = E; a.Epad = (E + 63) / 64 * 64; a.logits = logits;
-    dim3 grid(a.Epad / 64, n);
     const size_t lds = head_lds_bytes(n, H, E, false);
-    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, false>(a, grid, lds, st);
-    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, false>(a, grid, lds, st);
+    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, false>(a, 0, lds, st);
+    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, false>(a, 0, lds, st);
     return FERRITE_ERR_INVALID_ARG;
 }
 
