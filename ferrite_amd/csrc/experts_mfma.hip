@@ -195,8 +195,8 @@ struct MfmaArgs {
     const uint8_t* sh_codes;      // shared expert
     const uint8_t* sh_scales;
     size_t codes_per_expert, scales_per_expert;
-    const int32_t *unit_expert, *unit_row0, *unit_rows, *n_units;
-    int n, topk, n_experts, hidden, inter, shared_inter, act_ld, unit_cap;
+    const int32_t *unit_expert, *unit_row0, *unit_rows, *unit_first, *unit_count, *n_units;
+    int n, topk, n_experts, hidden, inter, shared_inter, act_ld, unit_cap, max_units;
     float limit;
 };
 
@@ -472,15 +472,23 @@ __device__ __forceinline__ void pf_mainloop(const PfCtx& c, u4v* lds, v4f (&acc)
 }
 
 // Block -> (unit, item group).  Hardware deals consecutive blocks round-robin over the 8 XCDs; the live work
-// (n_units * groups) is cut into 8 contiguous ranges, one per XCD, so that the blocks of one unit, and mostly
-// of one expert, share an L2.  Returns false for blocks without work.
-__device__ __forceinline__ bool pf_block_work(int n_units, int groups, int& u, int& ig) {
+// (n_units * groups) is cut into 8 contiguous ranges, one per XCD, so that the blocks of one expert share an L2.
+// Within a range the order is (expert, item group, unit of the expert): the 2-3 units of an expert that need the
+// same weight tiles are dispatched back to back, run in lockstep and fetch those tiles from HBM once (with the
+// units of an expert a whole item-group sweep apart, the second one found them evicted and HBM traffic doubled,
+// which is what bounded the kernel).  Returns false for blocks without work or with inconsistent tables.
+__device__ __forceinline__ bool pf_block_work(const MfmaArgs& a, int groups, int& u, int& ig) {
+    const int n_units = min(*a.n_units, a.max_units);
     const int total = n_units * groups, per_xcd = (total + 7) >> 3;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int v = xcd * per_xcd + slot;
     if (slot >= per_xcd || v >= total) return false;
-    u = v / groups;
-    ig = v - u * groups;
+    const int up = v / groups;                       // some unit of the expert whose segment holds v
+    const int first = a.unit_first[up], ne = a.unit_count[up];
+    if (first < 0 || ne < 1 || up < first || up >= first + ne || first + ne > n_units) return false;
+    const int vl = v - first * groups;               // 0 .. ne * groups - 1
+    ig = vl / ne;
+    u = first + (vl - ig * ne);
     return true;
 }
 
@@ -525,7 +533,7 @@ __global__ __launch_bounds__(256, 2) void gate_up_prefill_kernel(MfmaArgs a, int
                                                               uint8_t* __restrict__ act_s) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig;
-    if (!pf_block_work(*a.n_units, groups, u, ig)) return;
+    if (!pf_block_work(a, groups, u, ig)) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
@@ -594,7 +602,7 @@ __global__ __launch_bounds__(256, 2) void down_prefill_kernel(MfmaArgs a, int gr
                                                            const uint8_t* __restrict__ act_s, YT* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig;
-    if (!pf_block_work(*a.n_units, groups, u, ig)) return;
+    if (!pf_block_work(a, groups, u, ig)) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
@@ -649,12 +657,14 @@ static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int
     a.codes_per_expert = down ? L.dn_codes_per_expert : L.gu_codes_per_expert;
     a.scales_per_expert = down ? L.dn_scales_per_expert : L.gu_scales_per_expert;
     a.unit_expert = units.unit_expert; a.unit_row0 = units.unit_row0; a.unit_rows = units.unit_rows;
+    a.unit_first = units.unit_first; a.unit_count = units.unit_count;
     a.n_units = units.n_units;
     a.n = n; a.topk = s.topk; a.n_experts = s.n_experts; a.hidden = s.hidden; a.inter = s.inter;
     a.shared_inter = s.shared_inter;
     a.act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
     a.limit = s.swiglu_limit;
     a.unit_cap = units.unit_rows_cap;
+    a.max_units = units.max_units;
     return a;
 }
 

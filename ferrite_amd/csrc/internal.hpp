@@ -21,6 +21,8 @@ struct UnitTables {
     int32_t* unit_expert;  // [max_units] expert id (n_experts = the shared expert)
     int32_t* unit_row0;    // [max_units] first grouped row
     int32_t* unit_rows;    // [max_units] rows in the unit (1..unit_rows)
+    int32_t* unit_first;   // [max_units] index of the first unit of this unit's expert (may be NULL: not written)
+    int32_t* unit_count;   // [max_units] number of units of this unit's expert
     int32_t* n_units;      // [1]
     int unit_rows_cap;     // rows per unit (column tile of the GEMM)
     int max_units;

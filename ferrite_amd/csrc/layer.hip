@@ -29,7 +29,7 @@ int check_launch(const char* what) {
 // ---- workspace: fixed offsets for (shape, n, mode) ----
 struct Workspace {
     size_t logits, probs, ids_f32, ids, counts, starts, perm_map, gather_src, active, n_active;
-    size_t unit_expert, unit_row0, unit_rows, n_units, perm_scratch, perm_scratch_bytes, counters;
+    size_t unit_expert, unit_row0, unit_rows, unit_first, unit_count, n_units, perm_scratch, perm_scratch_bytes, counters;
     size_t xq, xs, act, act_s, y;
     size_t total;
     int max_units, rows, unit_cap;
@@ -78,6 +78,8 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     w.unit_expert = bump(off, (size_t)w.max_units * 4);
     w.unit_row0 = bump(off, (size_t)w.max_units * 4);
     w.unit_rows = bump(off, (size_t)w.max_units * 4);
+    w.unit_first = bump(off, (size_t)w.max_units * 4);
+    w.unit_count = bump(off, (size_t)w.max_units * 4);
     w.n_units = bump(off, 4);
     w.perm_scratch_bytes = ferrite_moe_permute_scratch_bytes(n, s.n_experts);
     w.perm_scratch = bump(off, w.perm_scratch_bytes);
@@ -201,7 +203,8 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     const int y_dtype = mode == FERRITE_MODE_MFMA_FP8 ? y_dtype_for(w.unit_cap) : FERRITE_DT_F32;
 
     UnitTables units{reinterpret_cast<int32_t*>(b + w.unit_expert), reinterpret_cast<int32_t*>(b + w.unit_row0),
-                     reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.n_units), w.unit_cap,
+                     reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.unit_first),
+                     reinterpret_cast<int32_t*>(b + w.unit_count), reinterpret_cast<int32_t*>(b + w.n_units), w.unit_cap,
                      w.max_units};
     uint8_t* xq = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xq) : nullptr;
     uint8_t* xs = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xs) : nullptr;

@@ -330,7 +330,7 @@ struct PermArgs {
     const int32_t* ids;
     int n, topk, n_experts;
     int32_t *counts, *starts, *perm_map, *gather_src, *active, *n_active;
-    int32_t *unit_expert, *unit_row0, *unit_rows, *n_units;
+    int32_t *unit_expert, *unit_row0, *unit_rows, *unit_first, *unit_count, *n_units;
     int unit_cap, max_units, has_shared;
 };
 
@@ -369,11 +369,13 @@ __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t*
             if (c > 0 && a.active) a.active[ract] = e;
             ract += c > 0;
             if (a.unit_cap > 0) {
+                const int first = rtile, cnt_e = (c + a.unit_cap - 1) / a.unit_cap;
                 for (int r = 0; r < c; r += a.unit_cap) {
                     if (rtile < a.max_units) {
                         a.unit_expert[rtile] = e;
                         a.unit_row0[rtile] = run + r;
                         a.unit_rows[rtile] = min(a.unit_cap, c - r);
+                        if (a.unit_first) { a.unit_first[rtile] = first; a.unit_count[rtile] = cnt_e; }
                     }
                     ++rtile;
                 }
@@ -397,6 +399,7 @@ __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t*
                 a.unit_expert[u] = E;
                 a.unit_row0[u] = a.n * a.topk + i * a.unit_cap;
                 a.unit_rows[u] = min(a.unit_cap, a.n - i * a.unit_cap);
+                if (a.unit_first) { a.unit_first[u] = total_tile; a.unit_count[u] = sh_tiles; }
             }
         }
         if (lane == 0) *a.n_units = min(total_tile + sh_tiles, a.max_units);
@@ -819,6 +822,7 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
     p.active = active; p.n_active = n_active; p.has_shared = s.shared_inter > 0;
     if (units) {
         p.unit_expert = units->unit_expert; p.unit_row0 = units->unit_row0; p.unit_rows = units->unit_rows;
+        p.unit_first = units->unit_first; p.unit_count = units->unit_count;
         p.n_units = units->n_units; p.unit_cap = units->unit_rows_cap; p.max_units = units->max_units;
     }
     const size_t lds = head_lds_bytes(n, s.hidden, s.n_experts, true);
@@ -1019,6 +1023,7 @@ int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* 
     a.active = active; a.n_active = n_active; a.has_shared = has_shared;
     if (units) {
         a.unit_expert = units->unit_expert; a.unit_row0 = units->unit_row0; a.unit_rows = units->unit_rows;
+        a.unit_first = units->unit_first; a.unit_count = units->unit_count;
         a.n_units = units->n_units; a.unit_cap = units->unit_rows_cap; a.max_units = units->max_units;
     }
     const int nchunk = (n + 63) / 64;
