@@ -170,6 +170,29 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
 
+    # A graph launch costs about 13 us on the device before its first kernel starts; a model runs all its layers
+    # from one graph, so the same layer is also timed eight times back to back inside one graph (reported as
+    # us_per_layer_in_stack; `value` stays the single-layer-per-launch figure).
+    us_in_stack = None
+    if trace is not None and n_layers == 1:
+        STACK = 8
+        hip.begin_capture()
+        for _ in range(STACK):
+            step()
+        stack_trace = hip.end_capture()
+        for _ in range(3):
+            hip.begin_verify(stack_trace)
+        hip.sync()
+        torch.cuda.synchronize()
+        reps = max(4, min(50, args.steps // 4))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            hip.begin_verify(stack_trace)
+        hip.sync()
+        torch.cuda.synchronize()
+        us_in_stack = (time.perf_counter() - t0) / reps / STACK * 1e6
+        hip.graph_destroy(stack_trace)
+
     # per-stage durations: eager launches with HIP events recorded on the launch stream between the stages
     ev = HipEvents()
     k_prof = min(args.steps, 50)
@@ -246,6 +269,7 @@ def main():
                    "launch": "eager" if trace is None else "hipGraph replay"},
         "layers_per_step": n_layers, "step_algorithmic_bytes": ab["total"] * n_layers,
         "us_per_layer": round(us_layer, 2), "us_per_layer_eager_events": round(eager_us, 2),
+        "us_per_layer_in_stack": None if us_in_stack is None else round(us_in_stack, 2),
         "stage_us": {k: round(v, 2) for k, v in stage_us.items()},
         "experts_hit": n_active, "max_tokens_per_expert": int(counts.max()),
         "max_over_mean_tokens_per_expert": round(float(counts.max() / max(counts.mean(), 1e-9)), 2),
