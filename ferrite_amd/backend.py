@@ -67,7 +67,7 @@ class WorkspaceView(C.Structure):
 
 
 EXPORTS = [
-    "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_matmul_f32",
+    "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_matmul_f32", "ferrite_rmsnorm_f32", "ferrite_hc_post_f32",
     "ferrite_swiglu_limited_f32", "ferrite_moe_route", "ferrite_moe_permute_scratch_bytes", "ferrite_moe_permute",
     "ferrite_mxfp4_dequant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes", "ferrite_moe_pack_weights",
     "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
@@ -88,6 +88,8 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_hip_last_error.restype = C.c_char_p
     lib.ferrite_matmul_f32.argtypes = [vp, vp, vp, vp, i32, i32, i32, vp]
     lib.ferrite_swiglu_limited_f32.argtypes = [vp, f32, vp, i32, i32, vp]
+    lib.ferrite_rmsnorm_f32.argtypes = [vp, vp, f32, vp, i32, i32, vp]
+    lib.ferrite_hc_post_f32.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, vp]
     lib.ferrite_moe_route.argtypes = [vp, vp, i32, i32, i32, i32, i32, f32, vp, vp, vp, vp]
     lib.ferrite_moe_permute_scratch_bytes.restype = sz
     lib.ferrite_moe_permute_scratch_bytes.argtypes = [i32, i32]
@@ -276,6 +278,38 @@ class HipBackend:
         self._enter()
         self._ck(self.lib.ferrite_matmul_f32(x.data_ptr(), w.data_ptr(), None if bias is None else bias.data_ptr(),
                                              out.data_ptr(), n, k, o, self._st()), "matmul")
+
+    def rmsnorm(self, x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor):
+        """lib.rs:76 / cpu.rs:124-143: x, out [..., dim] f32, w [dim] f32."""
+        self.recorder.record("rmsnorm")
+        self._leave()
+        if x.dim() < 1:
+            raise InvalidArg("rmsnorm rank 0")
+        dim = x.shape[-1]
+        if w.numel() != dim or tuple(out.shape) != tuple(x.shape):
+            raise InvalidArg("rmsnorm shape mismatch")
+        self._dev(x, torch.float32, "x"); self._dev(w, torch.float32, "w"); self._dev(out, torch.float32, "out")
+        self._enter()
+        self._ck(self.lib.ferrite_rmsnorm_f32(x.data_ptr(), w.data_ptr(), eps, out.data_ptr(), x.numel() // dim, dim,
+                                              self._st()), "rmsnorm")
+
+    def hc_post(self, x: torch.Tensor, residual: torch.Tensor, post: torch.Tensor, comb: torch.Tensor) -> torch.Tensor:
+        """lib.rs:256 / cpu.rs:788-807: x [s,h], residual [s,nh,h], post [s,nh], comb [s,nh,nh] -> new [s,nh,h]."""
+        self.recorder.record("hc_post")
+        self._leave()
+        if x.dim() != 2 or residual.dim() != 3:
+            raise InvalidArg("hc_post expects x [s,h] and residual [s,nh,h]")
+        s, h = x.shape
+        nh = residual.shape[1]
+        if tuple(residual.shape) != (s, nh, h) or tuple(post.shape) != (s, nh) or tuple(comb.shape) != (s, nh, nh):
+            raise ShapeMismatch("hc_post shape mismatch")
+        for t, nm in ((x, "x"), (residual, "residual"), (post, "post"), (comb, "comb")):
+            self._dev(t, torch.float32, nm)
+        out = torch.empty_like(residual)
+        self._enter()
+        self._ck(self.lib.ferrite_hc_post_f32(x.data_ptr(), residual.data_ptr(), post.data_ptr(), comb.data_ptr(),
+                                              out.data_ptr(), s, nh, h, self._st()), "hc_post")
+        return out
 
     def swiglu_limited(self, gate_up: torch.Tensor, limit: float, out: torch.Tensor):
         """lib.rs:83-85 / cpu.rs:178-203"""

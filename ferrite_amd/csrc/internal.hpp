@@ -97,6 +97,11 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
                      int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st);
 
+// block_ops.hip
+int launch_rmsnorm(const float* x, const float* w, float eps, float* out, int n, int dim, hipStream_t st);
+int launch_hc_post(const float* x, const float* residual, const float* post, const float* comb, float* out, int s,
+                   int nh, int h, hipStream_t st);
+
 // formats.hip
 int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, int operand_order,
                      hipStream_t st);

@@ -8,6 +8,7 @@
 // fe_expf restates that algorithm with every operation an individually rounded IEEE double operation, so the
 // device result is the same float.
 #pragma once
+#include <math.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -61,12 +62,14 @@ FE_HD double dadd(double a, double b) { return __dadd_rn(a, b); }
 FE_HD float fmul(float a, float b) { return __fmul_rn(a, b); }
 FE_HD float fadd(float a, float b) { return __fadd_rn(a, b); }
 FE_HD float fdiv(float a, float b) { return __fdiv_rn(a, b); }
+FE_HD float fsqrt(float a) { return __ocml_sqrt_f32(a); }   // correctly rounded (__fsqrt_rn is the native approximation)
 #else
 FE_HD double dmul(double a, double b) { volatile double r = a * b; return r; }
 FE_HD double dadd(double a, double b) { volatile double r = a + b; return r; }
 FE_HD float fmul(float a, float b) { volatile float r = a * b; return r; }
 FE_HD float fadd(float a, float b) { volatile float r = a + b; return r; }
 FE_HD float fdiv(float a, float b) { volatile float r = a / b; return r; }
+FE_HD float fsqrt(float a) { volatile float r = sqrtf(a); return r; }
 #endif
 
 // float exp, bit-identical to glibc >= 2.27 expf on x86-64 for finite results.

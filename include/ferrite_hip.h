@@ -166,6 +166,20 @@ int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_we
                             const void* x, int x_dtype, int n, void* out, int out_dtype, int mode,
                             void* workspace, size_t workspace_bytes, ferrite_stream_t stream);
 
+/* ---- the steps on either side of the layer (crates/ferrite-exec/src/lib.rs:487-492) ---- */
+
+/* KernelBackend::rmsnorm (crates/ferrite-kernel/src/lib.rs:76; CpuBackend, cpu.rs:124-143; CUDA: ferrite_rmsnorm,
+ * cuda.rs): x, out [n, dim] f32, w [dim] f32.  Bit-exact to the reference: the squares of a row are summed left to
+ * right in f32, inv = 1 / sqrt(ss / dim + eps), out = (x * inv) * w. */
+int ferrite_rmsnorm_f32(const float* x, const float* w, float eps, float* out, int n, int dim, ferrite_stream_t stream);
+
+/* KernelBackend::hc_post (lib.rs:256; cpu.rs:788-807; CUDA hc_post_kernel, kernels/cuda/ferrite_kernels.cu:2679):
+ * out[t,i,:] = post[t,i] * x[t,:] + sum_k comb[t,k,i] * residual[t,k,:] in k order, bit-exact.
+ * x [s,h], residual [s,nh,h], post [s,nh], comb [s,nh,nh], out [s,nh,h], all f32; nh <= 8, h % 4 == 0, 16-byte
+ * aligned x/residual/out, else FERRITE_DECLINED / FERRITE_ERR_INVALID_ARG. */
+int ferrite_hc_post_f32(const float* x, const float* residual, const float* post, const float* comb, float* out,
+                        int s, int nh, int h, ferrite_stream_t stream);
+
 /* The same layer with HIP events recorded on `stream` at the stage boundaries, the counterpart of the
  * reference's FERRITE_TIMING probes (crates/ferrite-exec/src/lib.rs:1184-1299).  stage_events_host is a host
  * array of FERRITE_MOE_STAGE_EVENTS hipEvent_t handles (any may be NULL): [0] before the router GEMM, then

@@ -72,6 +72,8 @@ def lib() -> C.CDLL:
         L.fo_dequant_fp4_row32.argtypes = [vp, vp, C.c_size_t, C.c_size_t, vp]
         L.fo_matmul.argtypes = [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]
         L.fo_swiglu_limited.argtypes = [vp, C.c_float, vp, C.c_int, C.c_int]
+        L.fo_rmsnorm.argtypes = [vp, vp, C.c_float, vp, C.c_int, C.c_int]
+        L.fo_hc_post.argtypes = [vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]
         L.fo_moe_route.argtypes = [vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, vp, vp]
         L.fo_moe_route_grouped.argtypes = [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, vp, vp]
         L.fo_expert_ffn.argtypes = [vp, vp, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int]
@@ -159,6 +161,29 @@ def swiglu_limited(gate_up, limit: float) -> np.ndarray:
         raise OracleError("swiglu last dim must be even")
     out = np.empty((n, two_i // 2), np.float32)
     _ck(lib().fo_swiglu_limited(_p(g), limit, _p(out), n, two_i // 2), "swiglu")
+    return out
+
+
+def rmsnorm(x, w, eps: float) -> np.ndarray:
+    """cpu.rs:124-143; x [n, dim], w [dim]."""
+    xv, wv = _f32(x), _f32(w)
+    n, dim = xv.shape
+    if wv.size != dim:
+        raise OracleError("rmsnorm shape mismatch")
+    out = np.empty_like(xv)
+    _ck(lib().fo_rmsnorm(_p(xv), _p(wv), eps, _p(out), n, dim), "rmsnorm")
+    return out
+
+
+def hc_post(x, residual, post, comb) -> np.ndarray:
+    """cpu.rs:788-807; x [s,h], residual [s,nh,h], post [s,nh], comb [s,nh,nh] -> [s,nh,h]."""
+    xv, rv, pv, cv = _f32(x), _f32(residual), _f32(post), _f32(comb)
+    s, h = xv.shape
+    nh = rv.shape[1]
+    if rv.shape != (s, nh, h) or pv.shape != (s, nh) or cv.shape != (s, nh, nh):
+        raise OracleError("hc_post shape mismatch")
+    out = np.empty_like(rv)
+    _ck(lib().fo_hc_post(_p(xv), _p(rv), _p(pv), _p(cv), _p(out), s, nh, h), "hc_post")
     return out
 
 

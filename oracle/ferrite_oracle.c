@@ -235,6 +235,48 @@ int fo_swiglu_limited(const float* gate_up, float limit, float* out, int n, int 
     return 0;
 }
 
+/* crates/ferrite-kernel/src/cpu.rs:124-143 (KernelBackend::rmsnorm, lib.rs:76): per row, the squares are summed left to
+ * right in f32 (Iterator::sum is a sequential fold; square and add are separately rounded), divided by the row length,
+ * inv = 1 / sqrt(ss + eps) with correctly rounded sqrt and division, out = (x * inv) * w. */
+int fo_rmsnorm(const float* x, const float* w, float eps, float* out, int n, int dim) {
+    if (n < 0 || dim <= 0) return 1;
+    for (int i = 0; i < n; ++i) {
+        const float* row = x + (size_t)i * dim;
+        float ss = 0.0f;
+        for (int j = 0; j < dim; ++j) {
+            float sq = row[j] * row[j];
+            ss = ss + sq;
+        }
+        ss = ss / (float)dim;
+        float inv = 1.0f / sqrtf(ss + eps);
+        for (int j = 0; j < dim; ++j) {
+            float t = row[j] * inv;
+            out[(size_t)i * dim + j] = t * w[j];
+        }
+    }
+    return 0;
+}
+
+/* crates/ferrite-kernel/src/cpu.rs:788-807 (KernelBackend::hc_post, lib.rs:256; same loop in
+ * crates/ferrite-exec/src/mhc.rs:195-213): out[t,i,:] = post[t,i] * x[t,:] + sum_k comb[t,k,i] * residual[t,k,:],
+ * accumulated in k order with separately rounded multiply and add.
+ * x [s,h], residual [s,nh,h], post [s,nh], comb [s,nh,nh], out [s,nh,h]. */
+int fo_hc_post(const float* x, const float* residual, const float* post, const float* comb, float* out, int s, int nh,
+               int h) {
+    if (s < 0 || nh <= 0 || h <= 0) return 1;
+    for (int t = 0; t < s; ++t)
+        for (int i = 0; i < nh; ++i)
+            for (int j = 0; j < h; ++j) {
+                float acc = post[(size_t)t * nh + i] * x[(size_t)t * h + j];
+                for (int k = 0; k < nh; ++k) {
+                    float p = comb[((size_t)t * nh + k) * nh + i] * residual[((size_t)t * nh + k) * h + j];
+                    acc = acc + p;
+                }
+                out[((size_t)t * nh + i) * h + j] = acc;
+            }
+    return 0;
+}
+
 typedef struct { float s; int j; } scored_t;
 
 /* cpu.rs:560: descending score, ties -> ascending index.  A strict total order, so any sort agrees

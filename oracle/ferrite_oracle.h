@@ -19,6 +19,10 @@
  *   fo_matmul / fo_swiglu_limited / fo_moe_route
  *       -> crates/ferrite-kernel/tests/golden.rs:14-27,44-55,189-210,
  *          gpu_smoke.rs:139-155 ramp fixture (closed form), brute force. PINNED
+ *   fo_rmsnorm / fo_hc_post (the steps before and after the layer)
+ *       -> golden.rs:30-42 closed form; no numeric vector for hc_post exists in the reference
+ *          (gpu_smoke.rs:308-348 compares device against CpuBackend), so it is pinned by a NumPy
+ *          statement with explicit f32 rounding, the identity-mix special case and linearity.  PINNED
  *   fo_moe_permute / fo_moe_align_host
  *       -> chain_dev.rs:25042-25061 vector, stable-sort closed form.     PINNED
  *   fo_moe_ffn_mxfp4 (f32 mode)
@@ -60,6 +64,11 @@ void    fo_dequant_fp4_row32(const uint8_t* w, const uint8_t* scale, size_t out,
 int fo_matmul(const float* x, const float* w, const float* bias, float* out, int n, int k, int o);
 /* cpu.rs:178-203. gate_up [n, 2*inter] (gate first), out [n, inter] */
 int fo_swiglu_limited(const float* gate_up, float limit, float* out, int n, int inter);
+/* cpu.rs:124-143 */
+int fo_rmsnorm(const float* x, const float* w, float eps, float* out, int n, int dim);
+/* cpu.rs:788-807: x [s,h], residual [s,nh,h], post [s,nh], comb [s,nh,nh], out [s,nh,h] */
+int fo_hc_post(const float* x, const float* residual, const float* post, const float* comb, float* out, int s, int nh,
+               int h);
 /* cpu.rs:528-572. probs/ids [n, topk]; ids as f32 like the reference. 2 = NaN score (reference panics) */
 int fo_moe_route(const float* logits, const float* bias, int n, int e, int topk, float routed_scaling,
                  float* probs, float* ids);

@@ -216,3 +216,56 @@ def test_pack_is_a_pure_permutation(hip, oracle):
                 w, s = getattr(inp, f"sh_{wn}_w")[0], getattr(inp, f"sh_{sn}_s")[0]
             got = host(hip, hip.packed_dequant(layer, e, which))
             assert np.array_equal(got, oracle.dequant_fp4_row32(w, s)), (e, which)
+
+
+# ---- the steps before and after the layer ----
+@pytest.mark.parametrize("n,dim", [(1, 4), (11, 4096), (3, 517), (5, 7168), (2, 9000)])
+def test_rmsnorm_bit_exact_vs_oracle(hip, oracle, n, dim):  # gpu_smoke.rs:56-70 shape [11, 4096] included
+    rng = np.random.default_rng(n * 1000 + dim)
+    x = (rng.standard_normal((n, dim)) * rng.uniform(1e-3, 30, (n, 1))).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, dim).astype(np.float32)
+    if dim == 4:
+        x[0] = [1., 2., 3., 4.]                       # golden.rs:30-42
+    out = torch.empty(n, dim, device=hip.device)
+    hip.rmsnorm(torch.from_numpy(x).to(hip.device), torch.from_numpy(w).to(hip.device), 1e-5, out)
+    hip.sync()
+    assert np.array_equal(out.cpu().numpy(), oracle.rmsnorm(x, w, 1e-5))
+
+
+def test_rmsnorm_sequential_sum_and_errors(hip, oracle):
+    from ferrite_amd.backend import InvalidArg
+    row = np.full((1, 4097), 2.0 ** -13, np.float32)   # the left-to-right f32 sum drops every small square
+    row[0, 0] = 1.0
+    w = np.ones(4097, np.float32)
+    out = torch.empty(1, 4097, device=hip.device)
+    hip.rmsnorm(torch.from_numpy(row).to(hip.device), torch.from_numpy(w).to(hip.device), 0.0, out)
+    hip.sync()
+    assert np.array_equal(out.cpu().numpy(), oracle.rmsnorm(row, w, 0.0))
+    with pytest.raises(InvalidArg):
+        hip.rmsnorm(torch.zeros(2, 8, device=hip.device), torch.zeros(7, device=hip.device), 1e-5,
+                    torch.zeros(2, 8, device=hip.device))
+
+
+@pytest.mark.parametrize("s,nh,h", [(2, 4, 64), (32, 4, 4096), (5, 2, 12), (3, 8, 7168)])
+def test_hc_post_bit_exact_vs_oracle(hip, oracle, s, nh, h):  # gpu_smoke.rs:308-348 shape (2, 4, 64) included
+    rng = np.random.default_rng(s * 100 + nh)
+    x = rng.standard_normal((s, h)).astype(np.float32)
+    res = rng.standard_normal((s, nh, h)).astype(np.float32)
+    post = rng.uniform(0, 2, (s, nh)).astype(np.float32)
+    comb = rng.uniform(0, 1, (s, nh, nh)).astype(np.float32)
+    if (s, nh, h) == (2, 4, 64):
+        x = ((np.arange(s * h) * 7 % 31) * 0.03).astype(np.float32).reshape(s, h)
+        res = ((np.arange(s * nh * h) * 13 % 47) * 0.02 - 0.5).astype(np.float32).reshape(s, nh, h)
+    d = lambda a: torch.from_numpy(a).to(hip.device)
+    out = hip.hc_post(d(x), d(res), d(post), d(comb))
+    hip.sync()
+    assert np.array_equal(out.cpu().numpy(), oracle.hc_post(x, res, post, comb))
+
+
+def test_hc_post_shape_errors(hip):
+    from ferrite_amd.backend import Declined, ShapeMismatch
+    z = lambda *sh: torch.zeros(*sh, device=hip.device)
+    with pytest.raises(ShapeMismatch):
+        hip.hc_post(z(2, 8), z(2, 4, 8), z(2, 3), z(2, 4, 4))
+    with pytest.raises(Declined):
+        hip.hc_post(z(2, 8), z(2, 9, 8), z(2, 9), z(2, 9, 9))     # more than 8 flows

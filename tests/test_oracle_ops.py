@@ -228,3 +228,85 @@ def test_moe_permute_out_of_range_ids_drop_out(oracle):  # dsv41_route.cu:253-26
     assert t["perm_map"].tolist() == [0, -1, -1, 1]
     assert t["gather_src"].tolist() == [0, 3, -1, -1]
     assert t["starts"][-1] == 2
+
+
+# ---- the steps before and after the layer: rmsnorm (cpu.rs:124-143), hc_post (cpu.rs:788-807) ----
+def _rmsnorm_f32_steps(x, w, eps):
+    """The reference's evaluation order, one rounded f32 operation at a time."""
+    f = np.float32
+    out = np.empty_like(x)
+    for i, row in enumerate(x):
+        ss = f(0.0)
+        for v in row:
+            ss = f(ss + f(v * v))
+        ss = f(ss / f(len(row)))
+        inv = f(f(1.0) / np.sqrt(f(ss + f(eps)), dtype=np.float32))
+        for j, v in enumerate(row):
+            out[i, j] = f(f(v * inv) * w[j])
+    return out
+
+
+def test_rmsnorm_manual(oracle):  # golden.rs:30-42
+    x = np.array([[1., 2., 3., 4.]], np.float32)
+    out = oracle.rmsnorm(x, np.ones(4, np.float32), 1e-6)
+    inv = np.float32(1.0) / np.sqrt(np.float32((1 + 4 + 9 + 16) / 4) + np.float32(1e-6), dtype=np.float32)
+    assert np.abs(out[0] - x[0] * inv).max() < 1e-5           # the reference test's own bar
+    assert np.array_equal(out, _rmsnorm_f32_steps(x, np.ones(4, np.float32), 1e-6))
+
+
+def test_rmsnorm_is_the_sequential_f32_evaluation(oracle):
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((3, 517)) * np.array([[1e-3], [1.0], [300.0]])).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 517).astype(np.float32)
+    got = oracle.rmsnorm(x, w, 1e-5)
+    assert np.array_equal(got, _rmsnorm_f32_steps(x, w, 1e-5))
+    # a row on which the left-to-right f32 sum differs from a pairwise or float64 sum: 1 followed by many 2^-13
+    # (each square 2^-26 is below half an ulp of 1 and is dropped one at a time, but not when summed first)
+    row = np.full((1, 4097), 2.0 ** -13, np.float32)
+    row[0, 0] = 1.0
+    seq = oracle.rmsnorm(row, np.ones(4097, np.float32), 0.0)
+    ss64 = np.float32(np.sum(row.astype(np.float64) ** 2) / 4097)
+    other = row * (np.float32(1.0) / np.sqrt(ss64, dtype=np.float32))
+    assert np.array_equal(seq, _rmsnorm_f32_steps(row, np.ones(4097, np.float32), 0.0))
+    assert not np.array_equal(seq, other)
+    # unit mean square once eps is negligible against the row's mean square (rows 1 and 2)
+    ms = np.mean(got[1:].astype(np.float64) ** 2 / w.astype(np.float64) ** 2, axis=1)
+    assert np.abs(ms - 1.0).max() < 1e-3
+    with pytest.raises(oracle.OracleError):
+        oracle.rmsnorm(x, w[:-1], 1e-5)
+
+
+def _hc_post_f32_steps(x, res, post, comb):
+    f = np.float32
+    s, nh, h = res.shape
+    out = np.empty_like(res)
+    for t in range(s):
+        for i in range(nh):
+            acc = (post[t, i] * x[t]).astype(f)
+            for k in range(nh):
+                acc = (acc + (comb[t, k, i] * res[t, k]).astype(f)).astype(f)
+            out[t, i] = acc
+    return out
+
+
+def test_hc_post_reference_fixture_and_special_cases(oracle):
+    # inputs of gpu_smoke.rs:337-343 (s=2, n=4, h=64); post/comb there come from hc_pre, any values pin the formula
+    s, nh, h = 2, 4, 64
+    x = ((np.arange(s * h) * 7 % 31) * 0.03).astype(np.float32).reshape(s, h)
+    res = ((np.arange(s * nh * h) * 13 % 47) * 0.02 - 0.5).astype(np.float32).reshape(s, nh, h)
+    rng = np.random.default_rng(9)
+    post = rng.uniform(0, 2, (s, nh)).astype(np.float32)          # sigmoid range of hc_pre (mhc.rs:252-255)
+    comb = rng.uniform(0, 1, (s, nh, nh)).astype(np.float32)
+    got = oracle.hc_post(x, res, post, comb)
+    assert got.shape == (s, nh, h)
+    assert np.array_equal(got, _hc_post_f32_steps(x, res, post, comb))
+    # the mix is comb[t, k, i] (column i), not comb[t, i, k]: a non-symmetric comb tells them apart
+    assert not np.array_equal(got, _hc_post_f32_steps(x, res, post, comb.transpose(0, 2, 1).copy()))
+    # identity mix and unit post: out[t, i] = x[t] + residual[t, i], exactly
+    eye = np.broadcast_to(np.eye(nh, dtype=np.float32), (s, nh, nh)).copy()
+    one = np.ones((s, nh), np.float32)
+    assert np.array_equal(oracle.hc_post(x, res, one, eye), x[:, None, :] + res)
+    # zero mix: out = post * x
+    assert np.array_equal(oracle.hc_post(x, res, post, np.zeros_like(comb)), post[:, :, None] * x[:, None, :])
+    with pytest.raises(oracle.OracleError):
+        oracle.hc_post(x, res, post[:, :2], comb)
