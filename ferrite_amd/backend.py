@@ -61,6 +61,11 @@ class MoeWeights(C.Structure):
     _fields_ = [(k, C.c_void_p) for k in _WEIGHT_FIELDS]
 
 
+class MoeBlockArgs(C.Structure):
+    _fields_ = [("norm_w", C.c_void_p), ("eps", C.c_float), ("residual", C.c_void_p), ("post", C.c_void_p),
+                ("comb", C.c_void_p), ("nh", C.c_int)]
+
+
 class WorkspaceView(C.Structure):
     _fields_ = [(k, C.c_void_p) for k in ("logits", "probs", "ids_f32", "ids", "counts", "starts", "perm_map",
                                           "gather_src", "active", "n_active", "y")]
@@ -70,7 +75,7 @@ EXPORTS = [
     "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_matmul_f32", "ferrite_rmsnorm_f32", "ferrite_hc_post_f32",
     "ferrite_swiglu_limited_f32", "ferrite_moe_route", "ferrite_moe_permute_scratch_bytes", "ferrite_moe_permute",
     "ferrite_mxfp4_dequant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes", "ferrite_moe_pack_weights",
-    "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
+    "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_block_workspace_bytes", "ferrite_moe_block_mxfp4", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
     "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_timed", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
     "ferrite_graph_destroy",
 ]
@@ -102,6 +107,10 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_moe_packed_dequant.argtypes = [C.POINTER(MoeShape), vp, i32, i32, vp, vp]
     lib.ferrite_moe_layer_workspace_bytes.restype = sz
     lib.ferrite_moe_layer_unit_rows.argtypes = [C.POINTER(MoeShape), i32, i32]
+    lib.ferrite_moe_block_workspace_bytes.restype = sz
+    lib.ferrite_moe_block_workspace_bytes.argtypes = [C.POINTER(MoeShape), i32, i32]
+    lib.ferrite_moe_block_mxfp4.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp, C.POINTER(MoeBlockArgs), i32,
+                                            vp, i32, vp, sz, vp]
     lib.ferrite_moe_layer_workspace_bytes.argtypes = [C.POINTER(MoeShape), i32, i32]
     lib.ferrite_moe_layer_workspace_init.argtypes = [C.POINTER(MoeShape), i32, i32, vp, sz, vp]
     lib.ferrite_moe_layer_workspace_view.argtypes = [C.POINTER(MoeShape), i32, i32, vp, C.POINTER(WorkspaceView)]
@@ -475,6 +484,48 @@ class HipBackend:
             self._ck(self.lib.ferrite_moe_layer_mxfp4(*args), "moe_layer_mxfp4")
         else:
             self._ck(self.lib.ferrite_moe_layer_mxfp4_timed(*args, stage_events), "moe_layer_mxfp4")
+
+    def block_workspace(self, layer: MoeLayer, n: int, mode: int) -> torch.Tensor:
+        key = ("block", n, mode)
+        if key not in layer._ws:
+            nbytes = self.lib.ferrite_moe_block_workspace_bytes(C.byref(layer.shape), n, mode)
+            if nbytes == 0:
+                raise InvalidArg("unsupported shape / mode")
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+            self._enter()
+            self._ck(self.lib.ferrite_moe_layer_workspace_init(C.byref(layer.shape), n, mode, ws.data_ptr(), nbytes,
+                                                               self._st()), "workspace_init")
+            self._leave()
+            layer._ws[key] = ws
+        return layer._ws[key]
+
+    def moe_block_mxfp4(self, layer: MoeLayer, li: torch.Tensor, norm_w: torch.Tensor, eps: float,
+                        residual: torch.Tensor, post: torch.Tensor, comb: torch.Tensor, out: torch.Tensor,
+                        mode: int = MODE_MFMA_FP8):
+        """The FFN half of a decoder layer (exec/lib.rs:487-492): rmsnorm -> MoE FFN -> hc_post, one call.
+        li [n,H] f32, residual/out [n,nh,H] f32, post [n,nh], comb [n,nh,nh]."""
+        self.recorder.record("moe_block_mxfp4")
+        self._leave()
+        cfg = layer.cfg
+        if li.dim() != 2 or li.shape[1] != cfg.hidden:
+            raise ShapeMismatch(f"li {tuple(li.shape)} vs hidden {cfg.hidden}")
+        n = li.shape[0]
+        nh = residual.shape[1] if residual.dim() == 3 else -1
+        if (tuple(residual.shape) != (n, nh, cfg.hidden) or tuple(out.shape) != (n, nh, cfg.hidden)
+                or tuple(post.shape) != (n, nh) or tuple(comb.shape) != (n, nh, nh) or norm_w.numel() != cfg.hidden):
+            raise ShapeMismatch("moe_block shape mismatch")
+        for t, nm in ((li, "li"), (norm_w, "norm_w"), (residual, "residual"), (post, "post"), (comb, "comb"),
+                      (out, "out")):
+            self._dev(t, torch.float32, nm)
+        if mode == MODE_MFMA_FP8 and layer.packed is None:
+            raise InvalidArg("layer has no packed weights")
+        ws = self.block_workspace(layer, n, mode)
+        blk = MoeBlockArgs(norm_w.data_ptr(), eps, residual.data_ptr(), post.data_ptr(), comb.data_ptr(), nh)
+        self._enter()
+        self._ck(self.lib.ferrite_moe_block_mxfp4(C.byref(layer.shape), C.byref(layer.weights),
+                                                  None if layer.packed is None else layer.packed.data_ptr(),
+                                                  li.data_ptr(), C.byref(blk), n, out.data_ptr(), mode, ws.data_ptr(),
+                                                  ws.numel(), self._st()), "moe_block_mxfp4")
 
     def workspace_view(self, layer: MoeLayer, n: int, mode: int) -> Dict[str, torch.Tensor]:
         """Typed views of the intermediates the last layer call left in its workspace."""

@@ -295,6 +295,36 @@ extern "C" int ferrite_moe_layer_mxfp4_timed(const ferrite_moe_shape* shape, con
                           stage_events);
 }
 
+// ---- rmsnorm -> layer -> hc_post (exec/lib.rs:487-492) ----
+static size_t block_extra(const ferrite_moe_shape& s, int n) { return ((size_t)n * s.hidden * 4 + 255) / 256 * 256; }
+
+extern "C" size_t ferrite_moe_block_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode) {
+    if (check_shape(shape, n, mode)) return 0;
+    return carve(*shape, n, mode).total + 2 * block_extra(*shape, n);
+}
+
+extern "C" int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
+                                       const uint8_t* packed, const float* li, const ferrite_moe_block_args* blk, int n,
+                                       float* out, int mode, void* workspace, size_t workspace_bytes,
+                                       ferrite_stream_t stream) {
+    int rc = check_shape(shape, n, mode);
+    if (rc) return rc;
+    if (!li || !blk || !out || !workspace || !blk->norm_w || !blk->residual || !blk->post || !blk->comb)
+        return FERRITE_ERR_INVALID_ARG;
+    if (blk->nh <= 0) return FERRITE_ERR_INVALID_ARG;
+    const ferrite_moe_shape& s = *shape;
+    const size_t layer_bytes = carve(s, n, mode).total, extra = block_extra(s, n);
+    if (workspace_bytes < layer_bytes + 2 * extra) return FERRITE_ERR_WORKSPACE;
+    char* b = static_cast<char*>(workspace);
+    float* hfn = reinterpret_cast<float*>(b + layer_bytes);
+    float* ffn_out = reinterpret_cast<float*>(b + layer_bytes + extra);
+    if ((rc = ferrite_rmsnorm_f32(li, blk->norm_w, blk->eps, hfn, n, s.hidden, stream))) return rc;
+    if ((rc = moe_layer_impl(shape, wts, packed, hfn, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
+                             layer_bytes, stream, nullptr)))
+        return rc;
+    return ferrite_hc_post_f32(ffn_out, blk->residual, blk->post, blk->comb, out, n, blk->nh, s.hidden, stream);
+}
+
 // ---- graph capture (ferrite_graph_begin/end/instantiate/launch, cuda.rs:284-287) ----
 extern "C" int ferrite_graph_begin(ferrite_stream_t stream) {
     hipError_t e = hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal);

@@ -57,6 +57,7 @@ struct HipBackend::Api {
 #define FN(name) decltype(&::name) name = nullptr
     FN(ferrite_kernel_build_id); FN(ferrite_kernel_abi_version); FN(ferrite_hip_last_error);
     FN(ferrite_matmul_f32); FN(ferrite_swiglu_limited_f32); FN(ferrite_moe_route);
+    FN(ferrite_rmsnorm_f32); FN(ferrite_hc_post_f32);
     FN(ferrite_moe_packed_bytes); FN(ferrite_moe_pack_weights);
     FN(ferrite_moe_layer_workspace_bytes); FN(ferrite_moe_layer_workspace_init); FN(ferrite_moe_layer_mxfp4);
     FN(ferrite_graph_begin); FN(ferrite_graph_end); FN(ferrite_graph_launch); FN(ferrite_graph_destroy);
@@ -71,6 +72,7 @@ HipBackend::HipBackend(const std::string& so_path, int device) : api_(new Api) {
     if (!api_->name) throw FerriteError(FerriteError::InvalidArg, "missing symbol " #name)
     LOAD(ferrite_kernel_build_id); LOAD(ferrite_kernel_abi_version); LOAD(ferrite_hip_last_error);
     LOAD(ferrite_matmul_f32); LOAD(ferrite_swiglu_limited_f32); LOAD(ferrite_moe_route);
+    LOAD(ferrite_rmsnorm_f32); LOAD(ferrite_hc_post_f32);
     LOAD(ferrite_moe_packed_bytes); LOAD(ferrite_moe_pack_weights);
     LOAD(ferrite_moe_layer_workspace_bytes); LOAD(ferrite_moe_layer_workspace_init); LOAD(ferrite_moe_layer_mxfp4);
     LOAD(ferrite_graph_begin); LOAD(ferrite_graph_end); LOAD(ferrite_graph_launch); LOAD(ferrite_graph_destroy);
@@ -137,6 +139,44 @@ void HipBackend::swiglu_limited(const Tensor& gate_up, float limit, Tensor& out)
                                         (int)(two_i / 2), stream_), "swiglu");
     sync();
     dout.download(out.data.data(), n * two_i * 2);
+}
+
+// cpu.rs:124-143: the last dimension is normalised; w has that many elements; out has x's shape
+void HipBackend::rmsnorm(const Tensor& x, const Tensor& w, float eps, Tensor& out) {
+    rec("rmsnorm");
+    if (x.shape.empty()) throw FerriteError(FerriteError::InvalidArg, "rmsnorm rank 0");
+    const size_t dim = x.shape.back(), n = x.numel() / dim;
+    if (w.numel() != dim || out.shape != x.shape) throw FerriteError(FerriteError::InvalidArg, "rmsnorm shape mismatch");
+    DevBuf dx(n * dim * 4), dw(dim * 4), dout(n * dim * 4);
+    dx.upload(x.data.data(), n * dim * 4);
+    dw.upload(w.data.data(), dim * 4);
+    ck(api_->ferrite_rmsnorm_f32(static_cast<const float*>(dx.ptr), static_cast<const float*>(dw.ptr), eps,
+                                 static_cast<float*>(dout.ptr), (int)n, (int)dim, stream_), "rmsnorm");
+    sync();
+    dout.download(out.data.data(), n * dim * 4);
+}
+
+// cpu.rs:788-807: x [s,h], residual [s,nh,h], post [s,nh], comb [s,nh,nh] -> [s,nh,h]
+Tensor HipBackend::hc_post(const Tensor& x, const Tensor& residual, const Tensor& post, const Tensor& comb) {
+    rec("hc_post");
+    check_2d(x, "hc_post x");
+    if (residual.shape.size() != 3) throw FerriteError(FerriteError::InvalidArg, "hc_post residual must be [s,nh,h]");
+    const size_t s = x.shape[0], h = x.shape[1], nh = residual.shape[1];
+    if (residual.shape != std::vector<size_t>{s, nh, h} || post.shape != std::vector<size_t>{s, nh} ||
+        comb.shape != std::vector<size_t>{s, nh, nh})
+        throw FerriteError(FerriteError::ShapeMismatch, "hc_post shape mismatch");
+    Tensor out = Tensor::zeros({s, nh, h});
+    DevBuf dx(s * h * 4), dr(s * nh * h * 4), dp(s * nh * 4), dc(s * nh * nh * 4), dout(s * nh * h * 4);
+    dx.upload(x.data.data(), s * h * 4);
+    dr.upload(residual.data.data(), s * nh * h * 4);
+    dp.upload(post.data.data(), s * nh * 4);
+    dc.upload(comb.data.data(), s * nh * nh * 4);
+    ck(api_->ferrite_hc_post_f32(static_cast<const float*>(dx.ptr), static_cast<const float*>(dr.ptr),
+                                 static_cast<const float*>(dp.ptr), static_cast<const float*>(dc.ptr),
+                                 static_cast<float*>(dout.ptr), (int)s, (int)nh, (int)h, stream_), "hc_post");
+    sync();
+    dout.download(out.data.data(), s * nh * h * 4);
+    return out;
 }
 
 void HipBackend::moe_route(const Tensor& logits, const Tensor& bias, size_t topk, float routed_scaling, Tensor& probs,

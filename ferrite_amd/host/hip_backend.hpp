@@ -90,6 +90,8 @@ class HipBackend {
     // ---- KernelBackend, the ops on the path (host tensors in, pre-allocated host tensors out) ----
     void matmul(const Tensor& x, const Tensor& w, const Tensor* bias, Tensor& out);                  // lib.rs:73
     void swiglu_limited(const Tensor& gate_up, float limit, Tensor& out);                            // lib.rs:83-85
+    void rmsnorm(const Tensor& x, const Tensor& w, float eps, Tensor& out);                          // lib.rs:76
+    Tensor hc_post(const Tensor& x, const Tensor& residual, const Tensor& post, const Tensor& comb); // lib.rs:256
     void moe_route(const Tensor& logits, const Tensor& bias, size_t topk, float routed_scaling, Tensor& probs,
                    Tensor& ids, int n_group = 1, int topk_group = 1);                                // lib.rs:194-206
 

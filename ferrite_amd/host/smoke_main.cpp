@@ -43,6 +43,35 @@ static void swiglu_clamps(HipBackend& b) {   // golden.rs:44-55
     CHECK(std::fabs(out.data[1] - 10.0f / (1.0f + std::exp(-10.0f))) < 1e-6f, "gate clamped to 10");
 }
 
+static void rmsnorm_manual(HipBackend& b) {   // golden.rs:30-42
+    Tensor x = t2(1, 4, {1, 2, 3, 4}), w = t2(1, 4, {1, 1, 1, 1}), out = Tensor::zeros({1, 4});
+    b.rmsnorm(x, w, 1e-6f, out);
+    const float mean_sq = (1.0f + 4.0f + 9.0f + 16.0f) / 4.0f, inv = 1.0f / std::sqrt(mean_sq + 1e-6f);
+    for (int i = 0; i < 4; ++i) CHECK(std::fabs(out.data[i] - x.data[i] * inv) < 1e-5f, "rmsnorm");
+}
+
+static void hc_post_vs_host_loop(HipBackend& b) {   // inputs of gpu_smoke.rs:337-343, loop of cpu.rs:788-807
+    const size_t s = 2, n = 4, h = 64;
+    Tensor x = Tensor::zeros({s, h}), res = Tensor::zeros({s, n, h}), post = Tensor::zeros({s, n}), comb = Tensor::zeros({s, n, n});
+    for (size_t i = 0; i < s * h; ++i) x.data[i] = (float)(i * 7 % 31) * 0.03f;
+    for (size_t i = 0; i < s * n * h; ++i) res.data[i] = (float)(i * 13 % 47) * 0.02f - 0.5f;
+    for (size_t i = 0; i < s * n; ++i) post.data[i] = 0.25f + 0.2f * (float)i;
+    for (size_t i = 0; i < s * n * n; ++i) comb.data[i] = (float)((i * 5 + 3) % 11) / 16.0f;
+    Tensor out = b.hc_post(x, res, post, comb);
+    bool same = out.shape == std::vector<size_t>{s, n, h};
+    for (size_t t = 0; t < s && same; ++t)
+        for (size_t i = 0; i < n; ++i)
+            for (size_t j = 0; j < h; ++j) {
+                volatile float acc = post.data[t * n + i] * x.data[t * h + j];
+                for (size_t k = 0; k < n; ++k) {
+                    volatile float p = comb.data[(t * n + k) * n + i] * res.data[(t * n + k) * h + j];
+                    acc = acc + p;
+                }
+                if (out.data[(t * n + i) * h + j] != acc) same = false;
+            }
+    CHECK(same, "hc_post bit-exact against the host loop");
+}
+
 static void moe_route_noaux_tc(HipBackend& b) {   // golden.rs:189-210 and gpu_smoke.rs:139-155
     Tensor logits = t2(1, 3, {1.0f, 2.0f, 0.5f}), bias = t2(1, 3, {0, 0, 0.5f});
     Tensor probs = Tensor::zeros({1, 2}), ids = Tensor::zeros({1, 2});
@@ -198,6 +227,8 @@ int main(int argc, char** argv) {
         std::printf("build id %s\n", b.build_id().c_str());
         matmul_matches_manual(b); std::printf("matmul ok\n"); std::fflush(stdout);
         swiglu_clamps(b); std::printf("swiglu ok\n"); std::fflush(stdout);
+        rmsnorm_manual(b); std::printf("rmsnorm ok\n"); std::fflush(stdout);
+        hc_post_vs_host_loop(b); std::printf("hc_post ok\n"); std::fflush(stdout);
         moe_route_noaux_tc(b); std::printf("moe_route ok\n"); std::fflush(stdout);
         moe_fused_parity(b); std::fflush(stdout);
         graph_capture_smoke(b); std::printf("graph ok\n");

@@ -180,6 +180,28 @@ int ferrite_rmsnorm_f32(const float* x, const float* w, float eps, float* out, i
 int ferrite_hc_post_f32(const float* x, const float* residual, const float* post, const float* comb, float* out,
                         int s, int nh, int h, ferrite_stream_t stream);
 
+/* The FFN half of a decoder layer in one call, the three statements of crates/ferrite-exec/src/lib.rs:487-492:
+ *     hfn     = rmsnorm(li, post_attention_layernorm.weight, eps)
+ *     ffn_out = moe_ffn(hfn)                       (ferrite_moe_layer_mxfp4 on f32 activations)
+ *     out     = hc_post(ffn_out, residual, post, comb)
+ * li [n, H] f32 (the mixed stream that hc_pre produced), out [n, nh, H] f32.  The workspace is the layer's followed by
+ * two [n, H] f32 buffers: size it with ferrite_moe_block_workspace_bytes and initialise it once with
+ * ferrite_moe_layer_workspace_init (which only touches the layer's part).  Same rules as the layer call: no
+ * allocation, no synchronisation, a launch sequence that depends only on (shape, n, mode), capturable. */
+typedef struct {
+    const float* norm_w;    /* [H] */
+    float eps;
+    const float* residual;  /* [n, nh, H] */
+    const float* post;      /* [n, nh] */
+    const float* comb;      /* [n, nh, nh] */
+    int nh;                 /* hyper-connection streams (hc_mult), <= 8 */
+} ferrite_moe_block_args;
+
+size_t ferrite_moe_block_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
+int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, const uint8_t* packed,
+                            const float* li, const ferrite_moe_block_args* blk, int n, float* out, int mode,
+                            void* workspace, size_t workspace_bytes, ferrite_stream_t stream);
+
 /* The same layer with HIP events recorded on `stream` at the stage boundaries, the counterpart of the
  * reference's FERRITE_TIMING probes (crates/ferrite-exec/src/lib.rs:1184-1299).  stage_events_host is a host
  * array of FERRITE_MOE_STAGE_EVENTS hipEvent_t handles (any may be NULL): [0] before the router GEMM, then

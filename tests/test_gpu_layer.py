@@ -228,6 +228,63 @@ def test_layer_error_paths(hip):
     hip.sync()
 
 
+def _block_case(cfg, seed):
+    """Inputs of the FFN half of a decoder layer around a seeded MoE layer: pre-norm stream, norm weight, the nh
+    hyper-connection streams and their post/comb mixes (post in (0,2), comb row-stochastic-ish as hc_pre makes them)."""
+    import dataclasses
+    inp = synth.make_inputs(cfg, seed=seed)
+    rng = np.random.default_rng(seed + 100)
+    n, H, nh = cfg.n, cfg.hidden, 4
+    li = (rng.standard_normal((n, H)) * 3.0).astype(np.float32)
+    norm_w = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    residual = rng.standard_normal((n, nh, H)).astype(np.float32)
+    post = rng.uniform(0.0, 2.0, (n, nh)).astype(np.float32)
+    comb = rng.uniform(0.0, 1.0, (n, nh, nh)).astype(np.float32)
+    comb /= comb.sum(axis=2, keepdims=True)
+    return inp, li, norm_w, residual, post, comb, dataclasses
+
+
+def _block_oracle(oracle, inp, dc, li, norm_w, eps, residual, post, comb, act_mode):
+    hfn = oracle.rmsnorm(li, norm_w, eps)
+    ffn = oracle.moe_ffn_mxfp4(dc.replace(inp, x=hfn), act_mode=act_mode, n_threads=8)
+    return oracle.hc_post(ffn["out"], residual, post, comb), hfn
+
+
+@pytest.mark.parametrize("n", [8, 40])
+def test_block_rmsnorm_layer_hc_post(hip, oracle, n):
+    """exec/lib.rs:487-492 as one call: rmsnorm -> MoE FFN -> hc_post.  The normalised activations are bit-exact, so
+    routing is; the output keeps the layer's bars (relative to max|ref|)."""
+    cfg = synth.CONFIGS["c0"].with_tokens(n)
+    inp, li, norm_w, residual, post, comb, dc = _block_case(cfg, seed=31)
+    layer = hip.load_moe_layer(inp)
+    d = lambda a: torch.from_numpy(a).to(hip.device)
+    out = torch.empty(n, 4, cfg.hidden, device=hip.device)
+    for mode, act_mode, tol in ((MODE_F32_CHECK, 0, TOL_F32), (MODE_MFMA_FP8, 1, TOL_MFMA)):
+        hip.moe_block_mxfp4(layer, d(li), d(norm_w), 1e-6, d(residual), d(post), d(comb), out, mode)
+        hip.sync()
+        ref, hfn = _block_oracle(oracle, inp, dc, li, norm_w, 1e-6, residual, post, comb, act_mode)
+        assert max_abs_rel(out.cpu().numpy(), ref) <= tol
+    # graph capture of the whole block, replayed on fresh data
+    li_s, res_s = d(li).clone(), d(residual).clone()
+    nw, po, co = d(norm_w), d(post), d(comb)
+    hip.moe_block_mxfp4(layer, li_s, nw, 1e-6, res_s, po, co, out, MODE_MFMA_FP8)
+    hip.sync()
+    hip.begin_capture()
+    hip.moe_block_mxfp4(layer, li_s, nw, 1e-6, res_s, po, co, out, MODE_MFMA_FP8)
+    trace = hip.end_capture()
+    for seed in (41, 42):
+        rng = np.random.default_rng(seed)
+        li2 = (rng.standard_normal(li.shape) * 2.0).astype(np.float32)
+        res2 = rng.standard_normal(residual.shape).astype(np.float32)
+        li_s.copy_(d(li2)); res_s.copy_(d(res2))
+        torch.cuda.synchronize()
+        hip.begin_verify(trace)
+        assert hip.end_verify()
+        ref, _ = _block_oracle(oracle, inp, dc, li2, norm_w, 1e-6, res2, post, comb, 1)
+        assert max_abs_rel(out.cpu().numpy(), ref) <= TOL_MFMA
+    hip.graph_destroy(trace)
+
+
 def test_layer_repeated_calls_same_workspace(hip, oracle):
     """The fused routing kernel keeps arrival counters in the workspace and must leave them cleared."""
     inp = synth.make_inputs(synth.CONFIGS["c0"].with_tokens(40), seed=3)
