@@ -193,6 +193,54 @@ def main():
         us_in_stack = (time.perf_counter() - t0) / reps / STACK * 1e6
         hip.graph_destroy(stack_trace)
 
+    # The FFN half of a decoder layer around the same layer (exec/lib.rs:487-492): rmsnorm -> layer -> hc_post as one
+    # captured call, and the two neighbours on their own (torch events on the backend's stream).
+    block = None
+    if trace is not None and n_layers == 1:
+        nh = 4
+        g = torch.Generator(device="cpu").manual_seed(1)
+        li = (torch.randn(n, cfg.hidden, generator=g) * 3.0).to(hip.device)
+        norm_w = (torch.rand(cfg.hidden, generator=g) + 0.5).to(hip.device)
+        residual = torch.randn(n, nh, cfg.hidden, generator=g).to(hip.device)
+        post = (torch.rand(n, nh, generator=g) * 2.0).to(hip.device)
+        comb = torch.softmax(torch.randn(n, nh, nh, generator=g), dim=2).to(hip.device)
+        bout = torch.empty(n, nh, cfg.hidden, device=hip.device)
+        hfn = torch.empty(n, cfg.hidden, device=hip.device)
+        for _ in range(3):
+            hip.moe_block_mxfp4(layer, li, norm_w, 1e-6, residual, post, comb, bout, MODE_MFMA_FP8)
+        hip.sync()
+        hip.begin_capture()
+        hip.moe_block_mxfp4(layer, li, norm_w, 1e-6, residual, post, comb, bout, MODE_MFMA_FP8)
+        btrace = hip.end_capture()
+        reps = max(10, min(200, args.steps))
+        for _ in range(3):
+            hip.begin_verify(btrace)
+        hip.sync()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            hip.begin_verify(btrace)
+        hip.sync()
+        torch.cuda.synchronize()
+        us_block = (time.perf_counter() - t0) / reps * 1e6
+        hip.graph_destroy(btrace)
+
+        def op_us(fn):
+            with torch.cuda.stream(hip.stream):
+                for _ in range(5):
+                    fn()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(hip.stream)
+                for _ in range(50):
+                    fn()
+                e1.record(hip.stream)
+            e1.synchronize()
+            return e0.elapsed_time(e1) / 50 * 1e3
+
+        block = {"us_per_block": round(us_block, 2), "hc_streams": nh,
+                 "rmsnorm_us": round(op_us(lambda: hip.rmsnorm(li, norm_w, 1e-6, hfn)), 2),
+                 "hc_post_us": round(op_us(lambda: hip.hc_post(hfn, residual, post, comb)), 2)}
+
     # per-stage durations: eager launches with HIP events recorded on the launch stream between the stages
     ev = HipEvents()
     k_prof = min(args.steps, 50)
@@ -279,7 +327,7 @@ def main():
         "layer_tflops": round(flops / (us_layer * 1e-6) / 1e12, 2),
         "mfma_frac_of_fp8_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP8_TFLOPS, 4),
         "mfma_frac_of_mxfp4_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP4_TFLOPS, 4),
-        "unit_rows": unit_rows, "roofline": roofline, "cpu_baseline": cpu, "setup_s": round(t_setup, 1), "build_id": hip.build_id,
+        "block_rmsnorm_layer_hc_post": block, "unit_rows": unit_rows, "roofline": roofline, "cpu_baseline": cpu, "setup_s": round(t_setup, 1), "build_id": hip.build_id,
     }
     if trace is not None:
         hip.graph_destroy(trace)

@@ -20,18 +20,72 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(const float* __restrict__ x
     __shared__ __align__(16) float sq[RN_CHUNK];
     const int lane = threadIdx.x;
     const float* row = x + (size_t)blockIdx.x * dim;
+    const bool vec4 = (dim & 3) == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
+                                           reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     float ss = 0.0f;
     for (int base = 0; base < dim; base += RN_CHUNK) {
         const int len = min(RN_CHUNK, dim - base);
         const int len4 = (len + 3) & ~3;
-        for (int j = lane; j < len4; j += 64) {
-            const float v = j < len ? row[base + j] : 0.0f;   // padding squares are +0: adding them changes nothing
-            sq[j] = fmul(v, v);
+        if (vec4) {
+            // all of the lane's loads of the chunk are issued before the first square is written (16 in flight)
+            const float4* r4 = reinterpret_cast<const float4*>(row + base);
+            float4 v[RN_CHUNK / 256];
+#pragma unroll
+            for (int q = 0; q < RN_CHUNK / 256; ++q) {
+                const int j4 = q * 64 + lane;
+                v[q] = j4 * 4 < len ? r4[j4] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int q = 0; q < RN_CHUNK / 256; ++q) {
+                const int j4 = q * 64 + lane;
+                if (j4 * 4 < len4)
+                    reinterpret_cast<float4*>(sq)[j4] =
+                        make_float4(fmul(v[q].x, v[q].x), fmul(v[q].y, v[q].y), fmul(v[q].z, v[q].z), fmul(v[q].w, v[q].w));
+            }
+        } else {
+#pragma unroll 8
+            for (int j = lane; j < len4; j += 64) {
+                const float v = j < len ? row[base + j] : 0.0f;   // padding squares are +0: adding them changes nothing
+                sq[j] = fmul(v, v);
+            }
         }
         __syncthreads();
+        // batches of eight 16-byte reads, one counted wait per batch (LDS returns in order: lgkmcnt(8) = everything
+        // but the batch just issued), 32 dependent adds per batch; without this the chain stalls on every read
         const float4* s4 = reinterpret_cast<const float4*>(sq);
-#pragma unroll 8
-        for (int j = 0; j < len4 / 4; ++j) {
+        const int nb = len4 / 32;   // full batches
+        float4 r[2][8];
+        if (nb > 0) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) r[0][j] = s4[j];
+        }
+        for (int b = 0; b < nb; b += 2) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int bb = b + half;
+                if (bb < nb) {
+                    if (bb + 1 < nb) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) r[half ^ 1][j] = s4[(bb + 1) * 8 + j];
+                        __builtin_amdgcn_sched_barrier(0);
+                        __builtin_amdgcn_s_waitcnt(0xC87F);
+                    } else {
+                        __builtin_amdgcn_sched_barrier(0);
+                        __builtin_amdgcn_s_waitcnt(0xC07F);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float4 p = r[half][j];
+                        ss = fadd(ss, p.x);
+                        ss = fadd(ss, p.y);
+                        ss = fadd(ss, p.z);
+                        ss = fadd(ss, p.w);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        for (int j = nb * 8; j < len4 / 4; ++j) {
             const float4 p = s4[j];
             ss = fadd(ss, p.x);
             ss = fadd(ss, p.y);
@@ -43,7 +97,17 @@ __global__ __launch_bounds__(64) void rmsnorm_kernel(const float* __restrict__ x
     ss = fdiv(ss, (float)dim);
     const float inv = fdiv(1.0f, fsqrt(fadd(ss, eps)));
     float* orow = out + (size_t)blockIdx.x * dim;
-    for (int j = lane; j < dim; j += 64) orow[j] = fmul(fmul(row[j], inv), w[j]);
+    if (vec4) {
+#pragma unroll 4
+        for (int j4 = lane; j4 < dim / 4; j4 += 64) {
+            const float4 v = reinterpret_cast<const float4*>(row)[j4], g = reinterpret_cast<const float4*>(w)[j4];
+            reinterpret_cast<float4*>(orow)[j4] = make_float4(fmul(fmul(v.x, inv), g.x), fmul(fmul(v.y, inv), g.y),
+                                                              fmul(fmul(v.z, inv), g.z), fmul(fmul(v.w, inv), g.w));
+        }
+    } else {
+#pragma unroll 8
+        for (int j = lane; j < dim; j += 64) orow[j] = fmul(fmul(row[j], inv), w[j]);
+    }
 }
 
 // KernelBackend::hc_post (cpu.rs:788-807; the CUDA counterpart is hc_post_kernel, kernels/cuda/ferrite_kernels.cu:2679):
