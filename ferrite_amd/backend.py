@@ -61,6 +61,11 @@ class MoeWeights(C.Structure):
     _fields_ = [(k, C.c_void_p) for k in _WEIGHT_FIELDS]
 
 
+class MoeExpertSrc(C.Structure):
+    _fields_ = [(k, C.c_void_p) for k in ("gate_w", "gate_s", "up_w", "up_s", "down_w", "down_s")] + \
+               [("gate_up_scale_pitch", C.c_int64), ("down_scale_pitch", C.c_int64)]
+
+
 class MoeBlockArgs(C.Structure):
     _fields_ = [("norm_w", C.c_void_p), ("eps", C.c_float), ("residual", C.c_void_p), ("post", C.c_void_p),
                 ("comb", C.c_void_p), ("nh", C.c_int)]
@@ -74,7 +79,8 @@ class WorkspaceView(C.Structure):
 EXPORTS = [
     "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_matmul_f32", "ferrite_rmsnorm_f32", "ferrite_hc_post_f32",
     "ferrite_swiglu_limited_f32", "ferrite_moe_route", "ferrite_moe_permute_scratch_bytes", "ferrite_moe_permute",
-    "ferrite_mxfp4_dequant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes", "ferrite_moe_pack_weights",
+    "ferrite_mxfp4_dequant", "ferrite_mxfp4_quant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes",
+    "ferrite_moe_pack_weights", "ferrite_moe_pack_expert", "ferrite_moe_pack_router",
     "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_block_workspace_bytes", "ferrite_moe_block_mxfp4", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
     "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_timed", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
     "ferrite_graph_destroy",
@@ -101,6 +107,9 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_moe_permute.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     lib.ferrite_mxfp4_dequant.argtypes = [vp, vp, i64, i64, vp, vp]
     lib.ferrite_act_quant_fp8.argtypes = [vp, i32, i64, i32, vp, vp, vp]
+    lib.ferrite_mxfp4_quant.argtypes = [vp, i32, i64, i64, vp, vp, vp]
+    lib.ferrite_moe_pack_expert.argtypes = [vp, i32, vp, vp, vp]
+    lib.ferrite_moe_pack_router.argtypes = [vp, vp, vp, vp]
     lib.ferrite_moe_packed_bytes.restype = sz
     lib.ferrite_moe_packed_bytes.argtypes = [C.POINTER(MoeShape)]
     lib.ferrite_moe_pack_weights.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp]
@@ -392,6 +401,41 @@ class HipBackend:
                                                 self._st()), "mxfp4_dequant")
         self._leave()
         return out
+
+    def mxfp4_quant(self, x: torch.Tensor):
+        """[rows, cols] f32 / bf16 -> (codes [rows, cols/2] u8, scales [rows, cols/32] u8), quant.rs:217-238."""
+        if x.dtype not in (torch.float32, torch.bfloat16) or x.dim() != 2 or not x.is_contiguous():
+            raise InvalidArg("x must be contiguous [rows, cols] f32 or bf16")
+        rows, cols = x.shape
+        if cols % 32:
+            raise InvalidArg("cols must be a multiple of 32")
+        self._dev(x, x.dtype, "x")
+        codes = torch.empty((rows, cols // 2), dtype=torch.uint8, device=self.device)
+        s = torch.empty((rows, cols // 32), dtype=torch.uint8, device=self.device)
+        self._enter()
+        self._ck(self.lib.ferrite_mxfp4_quant(x.data_ptr(), DT_F32 if x.dtype == torch.float32 else DT_BF16, rows,
+                                              cols, codes.data_ptr(), s.data_ptr(), self._st()), "mxfp4_quant")
+        self._leave()
+        return codes, s
+
+    def pack_expert(self, layer: MoeLayer, expert: int, gate=None, up=None, down=None, gate_up_scale_pitch: int = 0,
+                    down_scale_pitch: int = 0):
+        """Repack one expert's matrices into layer.packed: gate / up / down are (codes, scales) pairs of device
+        uint8 tensors in the checkpoint layout, or None to leave that group as it is."""
+        src = MoeExpertSrc()
+        keep = []
+        for key, pair in (("gate", gate), ("up", up), ("down", down)):
+            if pair is None:
+                continue
+            w, s = pair
+            self._dev(w, torch.uint8, key + " codes"); self._dev(s, torch.uint8, key + " scales")
+            setattr(src, key + "_w", w.data_ptr()); setattr(src, key + "_s", s.data_ptr())
+            keep += [w, s]
+        src.gate_up_scale_pitch, src.down_scale_pitch = gate_up_scale_pitch, down_scale_pitch
+        self._enter()
+        self._ck(self.lib.ferrite_moe_pack_expert(C.byref(layer.shape), expert, C.byref(src), layer.packed.data_ptr(),
+                                                  self._st()), "pack_expert")
+        self._leave()
 
     def act_quant_fp8(self, x: torch.Tensor):
         if x.dtype not in (torch.float32, torch.bfloat16) or x.dim() != 2 or not x.is_contiguous():

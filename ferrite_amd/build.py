@@ -55,20 +55,27 @@ def build(verbose: bool = False) -> str:
 
 HOST_DIR = os.path.join(HERE, "host")
 HOST_SMOKE = os.path.join(HOST_DIR, "hip_backend_smoke")
+HOST_SO = os.path.join(HOST_DIR, "libferrite_host.so")
 
 
 def build_host(verbose: bool = False) -> str:
     """Compile the C++ host side (HipBackend over the C ABI) and its smoke driver with g++."""
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
-    cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include", "-o", HOST_SMOKE,
-           os.path.join(HOST_DIR, "hip_backend.cpp"), os.path.join(HOST_DIR, "smoke_main.cpp"),
-           f"-L{rocm}/lib", "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm}/lib"]
-    if verbose:
-        print(" ".join(cmd))
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        sys.stderr.write(res.stdout + res.stderr)
-        raise RuntimeError("g++ failed (host side)")
+    common = ["g++", "-O2", "-std=c++17", "-Wall", "-pthread", "-D__HIP_PLATFORM_AMD__", f"-I{rocm}/include"]
+    libs = [f"-L{rocm}/lib", "-lamdhip64", "-ldl", f"-Wl,-rpath,{rocm}/lib"]
+    src = lambda *names: [os.path.join(HOST_DIR, n) for n in names]
+    cmds = [
+        common + ["-o", HOST_SMOKE] + src("hip_backend.cpp", "checkpoint.cpp", "smoke_main.cpp") + libs,
+        # the same host code as a shared library with a C facade, for bindings (ctypes) that cannot call C++
+        common + ["-fPIC", "-shared", "-o", HOST_SO] + src("hip_backend.cpp", "checkpoint.cpp", "host_capi.cpp") + libs,
+    ]
+    for cmd in cmds:
+        if verbose:
+            print(" ".join(cmd))
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            sys.stderr.write(res.stdout + res.stderr)
+            raise RuntimeError("g++ failed (host side)")
     return HOST_SMOKE
 
 

@@ -54,6 +54,7 @@ struct PackSrc {
     const uint8_t* scales[2];
     int rows, K;       // rows per matrix, columns
     int nmat, rpi;
+    size_t s_pitch;    // bytes between scale rows of the source (K/32 when dense; a loader may pad rows)
 };
 
 __global__ __launch_bounds__(256) void pack_codes_kernel(PackSrc s, int n_experts, uint4* __restrict__ dst) {
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(256) void pack_scales_kernel(PackSrc s, int n_exper
     const int tpm = 4 / s.nmat;
     int mat = tile / tpm;
     size_t row = item * s.rpi + (size_t)(tile % tpm) * 16 + (lane & 15);
-    const uint8_t* src = s.scales[mat] + (e * s.rows + row) * (s.K / 32);
+    const uint8_t* src = s.scales[mat] + (e * s.rows + row) * s.s_pitch;
     uint32_t v = 0;
     for (int q = 0; q < 4; ++q) {
         size_t kt = k4 * 4 + q;
@@ -757,17 +758,73 @@ extern "C" int ferrite_moe_pack_weights(const ferrite_moe_shape* shape, const fe
     hipStream_t st = as_stream(stream);
     if ((rc = launch_router_transpose(w->router_w, s.n_experts, s.hidden, reinterpret_cast<float*>(packed + L.router_t), st)))
         return rc;
-    PackSrc gu{{w->gate_w, w->up_w}, {w->gate_s, w->up_s}, s.inter, s.hidden, 2, 32};
+    PackSrc gu{{w->gate_w, w->up_w}, {w->gate_s, w->up_s}, s.inter, s.hidden, 2, 32, (size_t)s.hidden / 32};
     if ((rc = pack_one(gu, s.n_experts, packed + L.gu_codes, packed + L.gu_scales, st))) return rc;
-    PackSrc dn{{w->down_w, nullptr}, {w->down_s, nullptr}, s.hidden, s.inter, 1, 64};
+    PackSrc dn{{w->down_w, nullptr}, {w->down_s, nullptr}, s.hidden, s.inter, 1, 64, (size_t)s.inter / 32};
     if ((rc = pack_one(dn, s.n_experts, packed + L.dn_codes, packed + L.dn_scales, st))) return rc;
     if (s.shared_inter > 0) {
-        PackSrc sgu{{w->sh_gate_w, w->sh_up_w}, {w->sh_gate_s, w->sh_up_s}, s.shared_inter, s.hidden, 2, 32};
+        PackSrc sgu{{w->sh_gate_w, w->sh_up_w}, {w->sh_gate_s, w->sh_up_s}, s.shared_inter, s.hidden, 2, 32,
+                    (size_t)s.hidden / 32};
         if ((rc = pack_one(sgu, 1, packed + L.sh_gu_codes, packed + L.sh_gu_scales, st))) return rc;
-        PackSrc sdn{{w->sh_down_w, nullptr}, {w->sh_down_s, nullptr}, s.hidden, s.shared_inter, 1, 64};
+        PackSrc sdn{{w->sh_down_w, nullptr}, {w->sh_down_s, nullptr}, s.hidden, s.shared_inter, 1, 64,
+                    (size_t)s.shared_inter / 32};
         if ((rc = pack_one(sdn, 1, packed + L.sh_dn_codes, packed + L.sh_dn_scales, st))) return rc;
     }
     return FERRITE_OK;
+}
+
+// One expert at a time, for a loader that streams a checkpoint: the same kernels on a single expert's matrices,
+// written at that expert's place in the packed buffer.
+extern "C" int ferrite_moe_pack_expert(const ferrite_moe_shape* shape, int expert, const ferrite_moe_expert_src* src,
+                                       uint8_t* packed, ferrite_stream_t stream) {
+    int rc = check_shape_mfma(shape);
+    if (rc) return rc;
+    const ferrite_moe_shape& s = *shape;
+    if (!src || !packed || expert < 0 || expert > s.n_experts) return FERRITE_ERR_INVALID_ARG;
+    const bool shared = expert == s.n_experts;
+    if (shared && s.shared_inter == 0) return FERRITE_ERR_INVALID_ARG;
+    const bool has_gu = src->gate_w || src->gate_s || src->up_w || src->up_s;
+    const bool has_dn = src->down_w || src->down_s;
+    if (!has_gu && !has_dn) return FERRITE_ERR_INVALID_ARG;
+    if (has_gu && (!src->gate_w || !src->gate_s || !src->up_w || !src->up_s)) return FERRITE_ERR_INVALID_ARG;
+    if (has_dn && (!src->down_w || !src->down_s)) return FERRITE_ERR_INVALID_ARG;
+    const int inter = shared ? s.shared_inter : s.inter;
+    const size_t gu_pitch = src->gate_up_scale_pitch ? (size_t)src->gate_up_scale_pitch : (size_t)s.hidden / 32;
+    const size_t dn_pitch = src->down_scale_pitch ? (size_t)src->down_scale_pitch : (size_t)inter / 32;
+    if (src->gate_up_scale_pitch < 0 || src->down_scale_pitch < 0 || gu_pitch < (size_t)s.hidden / 32 ||
+        dn_pitch < (size_t)inter / 32)
+        return FERRITE_ERR_INVALID_ARG;
+    auto misaligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+    if (misaligned(src->gate_w) || misaligned(src->up_w) || misaligned(src->down_w) || misaligned(packed))
+        return FERRITE_DECLINED;
+    PackedLayout L = packed_layout(s);
+    hipStream_t st = as_stream(stream);
+    auto kt4 = [](size_t K) { return (K / 128 + 3) / 4; };
+    if (has_gu) {
+        const size_t cpe = (size_t)inter * s.hidden, spe = (size_t)(inter / 32) * kt4(s.hidden) * 1024;
+        PackSrc gu{{src->gate_w, src->up_w}, {src->gate_s, src->up_s}, inter, s.hidden, 2, 32, gu_pitch};
+        uint8_t* cd = packed + (shared ? L.sh_gu_codes : L.gu_codes + (size_t)expert * cpe);
+        uint8_t* sd = packed + (shared ? L.sh_gu_scales : L.gu_scales + (size_t)expert * spe);
+        if ((rc = pack_one(gu, 1, cd, sd, st))) return rc;
+    }
+    if (has_dn) {
+        const size_t cpe = (size_t)s.hidden * inter / 2, spe = (size_t)(s.hidden / 64) * kt4(inter) * 1024;
+        PackSrc dn{{src->down_w, nullptr}, {src->down_s, nullptr}, s.hidden, inter, 1, 64, dn_pitch};
+        uint8_t* cd = packed + (shared ? L.sh_dn_codes : L.dn_codes + (size_t)expert * cpe);
+        uint8_t* sd = packed + (shared ? L.sh_dn_scales : L.dn_scales + (size_t)expert * spe);
+        if ((rc = pack_one(dn, 1, cd, sd, st))) return rc;
+    }
+    return FERRITE_OK;
+}
+
+extern "C" int ferrite_moe_pack_router(const ferrite_moe_shape* shape, const float* router_w, uint8_t* packed,
+                                       ferrite_stream_t stream) {
+    int rc = check_shape_mfma(shape);
+    if (rc) return rc;
+    if (!router_w || !packed) return FERRITE_ERR_INVALID_ARG;
+    PackedLayout L = packed_layout(*shape);
+    return launch_router_transpose(router_w, shape->n_experts, shape->hidden,
+                                   reinterpret_cast<float*>(packed + L.router_t), as_stream(stream));
 }
 
 // dequantise one matrix out of the packed buffer (verification of the permutation)

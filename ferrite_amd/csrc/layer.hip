@@ -170,7 +170,8 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                           size_t workspace_bytes, ferrite_stream_t stream, void* const* ev) {
     int rc = check_shape(shape, n, mode);
     if (rc) return rc;
-    if (!wts || !wts->router_w || !x || !out || !workspace) return FERRITE_ERR_INVALID_ARG;
+    // the packed buffer carries the router weight (transposed); the checkpoint-layout one is read only without it
+    if (!wts || (!packed && !wts->router_w) || !x || !out || !workspace) return FERRITE_ERR_INVALID_ARG;
     if ((reinterpret_cast<uintptr_t>(workspace) & 255) || (reinterpret_cast<uintptr_t>(x) & 15) ||
         (reinterpret_cast<uintptr_t>(out) & 15))
         return FERRITE_ERR_INVALID_ARG;
@@ -236,8 +237,10 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         PackedLayout L = packed_layout(s);
         rc = launch_router_chain(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), n, s.hidden,
                                  s.n_experts, logits, st);
-        if (rc == FERRITE_DECLINED)
+        if (rc == FERRITE_DECLINED) {
+            if (!wts->router_w) return FERRITE_ERR_INVALID_ARG;   // this shape needs the checkpoint-layout router
             rc = launch_matmul_exact(x, x_dtype, wts->router_w, nullptr, logits, n, s.hidden, s.n_experts, st);
+        }
     } else {
         rc = launch_matmul_exact(x, x_dtype, wts->router_w, nullptr, logits, n, s.hidden, s.n_experts, st);
     }
@@ -338,7 +341,7 @@ extern "C" int ferrite_graph_end(ferrite_stream_t stream, void** graph_exec_out)
     if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture");
     hipGraphExec_t exec = nullptr;
     e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-    hipGraphDestroy(graph);
+    (void)hipGraphDestroy(graph);
     if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
     *graph_exec_out = exec;
     return FERRITE_OK;

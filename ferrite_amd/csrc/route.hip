@@ -159,7 +159,6 @@ __global__ void swiglu_kernel(const float* __restrict__ gate_up, float limit, fl
 // Semantics and operation order follow cpu.rs:546-569; ties -> lower index (cpu.rs:560).
 // ------------------------------------------------------------------------------------------------
 constexpr int RT_MAX_E = 512;
-constexpr int RT_NI = RT_MAX_E / 64;
 constexpr int RT_MAX_K = 32;
 
 __device__ __forceinline__ uint32_t ordered_u32(float f) {

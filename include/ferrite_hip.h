@@ -83,6 +83,12 @@ int ferrite_moe_permute(const int32_t* ids, int n, int topk, int n_experts, int3
 int ferrite_mxfp4_dequant(const uint8_t* w, const uint8_t* scale, int64_t rows, int64_t cols, float* dst,
                           ferrite_stream_t stream);
 
+/* f32 / bf16 -> MXFP4 (quant.rs:217-238 act_quant_fp4 with block 32 and the power-of-two scale of :190-198):
+ * x [rows, cols] -> codes [rows, cols/2] u8 (low nibble = even column), scale [rows, cols/32] e8m0 bytes.
+ * For checkpoints that keep their experts unquantised (crates/ferrite-model/src/weights.rs:133-149). */
+int ferrite_mxfp4_quant(const void* x, int x_dtype, int64_t rows, int64_t cols, uint8_t* codes, uint8_t* scale,
+                        ferrite_stream_t stream);
+
 /* Activation quantisation (quant.rs:190-214, block 32, power-of-two scale): x [rows, cols] (f32 or bf16) ->
  * q [rows, cols] e4m3 codes, scale [rows, cols/32] e8m0 bytes (2^(b-127)). */
 int ferrite_act_quant_fp8(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale,
@@ -121,6 +127,24 @@ typedef struct ferrite_moe_weights {
 size_t ferrite_moe_packed_bytes(const ferrite_moe_shape* shape);
 int ferrite_moe_pack_weights(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, uint8_t* packed,
                              ferrite_stream_t stream);
+/* The same repack one expert at a time, for a loader that walks a checkpoint whose experts are separate tensors
+ * (`{layer}.ffn.experts.{e}.w1|w2|w3.{weight,scale}`, crates/ferrite-models/src/dsv41/weights.rs:336-341) and
+ * stages them one by one: `expert` in [0, n_experts), or n_experts for the shared expert.  gate/up (w1/w3) go
+ * together, down (w2) on its own; either group may be left NULL.  The scale pitches are bytes between scale rows
+ * of the source, 0 = dense (cols/32): a loader that pads scale rows (weights.rs:599 sf_plane_pitch, the fix for the
+ * 10-byte w2 rows of kernels/cuda/dsv41_experts_mxf4.cu:121-168) passes its padded pitch; the packed layout itself
+ * has no row pitch, its scales sit in operand order.  Sources are device-accessible memory, codes 16-byte aligned. */
+typedef struct ferrite_moe_expert_src {
+    const uint8_t *gate_w, *gate_s, *up_w, *up_s; /* [I, H/2], [I, pitch] */
+    const uint8_t *down_w, *down_s;               /* [H, I/2], [H, pitch] */
+    int64_t gate_up_scale_pitch, down_scale_pitch;
+} ferrite_moe_expert_src;
+int ferrite_moe_pack_expert(const ferrite_moe_shape* shape, int expert, const ferrite_moe_expert_src* src,
+                            uint8_t* packed, ferrite_stream_t stream);
+/* The router's part of the packed buffer (the k-blocked transpose of router_w [E, H] f32). */
+int ferrite_moe_pack_router(const ferrite_moe_shape* shape, const float* router_w, uint8_t* packed,
+                            ferrite_stream_t stream);
+
 /* Inverse view for verification: dequantise matrix `which` (0 gate, 1 up, 2 down) of expert `expert`
  * (expert == n_experts selects the shared expert) from the packed buffer to f32 [rows, cols]. */
 int ferrite_moe_packed_dequant(const ferrite_moe_shape* shape, const uint8_t* packed, int expert, int which,
@@ -159,7 +183,9 @@ int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int 
                                      ferrite_moe_workspace_view* view_host);
 
 /* The layer.  x [n, H] (x_dtype), out [n, H] (out_dtype).  mode FERRITE_MODE_F32_CHECK reads `w` (checkpoint
- * layout) and requires f32 x; FERRITE_MODE_MFMA_FP8 reads `packed` (+ w->router_w / router_bias).
+ * layout) and requires f32 x; FERRITE_MODE_MFMA_FP8 reads `packed` and w->router_bias.  `packed` carries the
+ * router weight, so w->router_w may be NULL with it; the few shapes whose router falls back to the checkpoint
+ * layout (n > 65535, very large hidden) then return FERRITE_ERR_INVALID_ARG.
  * The launch sequence depends only on (shape, n, mode), never on the routing, so a captured graph of it
  * replays correctly for any input (the GraphCapable contract, crates/ferrite-kernel/src/graph.rs:48-64). */
 int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, const uint8_t* packed,
