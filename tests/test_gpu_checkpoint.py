@@ -147,10 +147,13 @@ def test_mxfp4_quant_bit_exact_vs_oracle(hip, oracle, dtype):
     assert np.array_equal(host(hip, codes).ravel(), co)
     sb = host(hip, s).ravel()
     assert sb.min() >= 1 and np.array_equal(np.exp2(sb.astype(np.float64) - 127), so.astype(np.float64))
-    # the quantised weights read back through the dequantiser are within half a grid step of the input
+    # read back through the dequantiser, every value is within half the widest grid spacing (2, from 4 to 6) of
+    # its input; the 3e38 block is left out, where 4 * 2^126 is beyond f32
     back = host(hip, hip.mxfp4_dequant(codes, s))
-    step = np.repeat(so.reshape(48, 8), 32, axis=1) * 1.0        # largest spacing of the grid is 2 (4 -> 6)
-    assert np.all(np.abs(back - xr) <= step + 1e-30)
+    half_step = np.repeat(so.reshape(48, 8), 32, axis=1).astype(np.float64)
+    ok = np.abs(back.astype(np.float64) - xr) <= half_step
+    ok[5, 0:32] = True
+    assert ok.all()
 
 
 def _glm_values(cfg, prefix, seed, as_bf16):
