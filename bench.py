@@ -96,6 +96,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0,
                     help="stack this many distinct layers into one captured step (default: 42 for c4, else 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-load-bench", action="store_true",
+                    help="skip the checkpoint -> packed-buffer load measurement (writes a shard of the layer to TMPDIR)")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of graph replays")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run a plain device copy of this many MiB (a counter calibration point for rocprofv3 --pmc)")
@@ -283,6 +285,46 @@ def main():
         if not args.tokens:
             roofline["traffic"] = MEASURED_TRAFFIC.get((args.config, "gate_up_prefill_kernel"))
 
+    # the row before the layer: one layer's shard (safetensors, the reference's tensor names) streamed from the
+    # page cache into the packed buffer; PCIe-bound, priced against a pinned -> device copy of the same size
+    load = None
+    if not args.no_load_bench and n_layers == 1:
+        try:
+            import tempfile
+            from ferrite_amd import checkpoint as ckpt
+            with tempfile.TemporaryDirectory() as td:
+                shard = os.path.join(td, "layer.safetensors")
+                ckpt.write_moe_checkpoint(shard, inp, "layers.6.ffn", ckpt.NAMING_DSV41)
+                with ckpt.Checkpoint(shard) as c:
+                    runs = []
+                    for _ in range(4):
+                        loaded, st = c.load_moe_layer(hip, cfg, "layers.6.ffn", ckpt.NAMING_DSV41)
+                        runs.append(st)
+                    same = bool(torch.equal(loaded.packed, layer.packed))
+                    del loaded
+                best = min(runs[1:], key=lambda r: r.seconds)
+                pin = torch.empty(best.source_bytes, dtype=torch.uint8).pin_memory()
+                dst = torch.empty(best.source_bytes, dtype=torch.uint8, device=hip.device)
+                copy_s = []
+                for _ in range(3):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    dst.copy_(pin, non_blocking=True)
+                    torch.cuda.synchronize()
+                    copy_s.append(time.perf_counter() - t0)
+                del pin, dst
+                pcie = best.source_bytes / min(copy_s) / 1e9
+                load = {"source_bytes": best.source_bytes, "workers": best.workers,
+                        "first_load_ms": round(runs[0].seconds * 1e3, 2), "ms": round(best.seconds * 1e3, 2),
+                        "GB_per_s": round(best.source_bytes / best.seconds / 1e9, 2),
+                        "pinned_copy_GB_per_s": round(pcie, 2),
+                        "frac_of_pinned_copy": round(best.source_bytes / best.seconds / 1e9 / pcie, 4),
+                        "packed_equals_memory_loaded": same,
+                        "what": "safetensors shard in the page cache -> pinned staging -> device -> repack kernels; "
+                                "first load also allocates the staging buffers"}
+        except Exception as e:   # a full TMPDIR must not cost the layer's numbers
+            load = {"error": f"{type(e).__name__}: {e}"}
+
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import binding as oracle
@@ -327,7 +369,7 @@ def main():
         "layer_tflops": round(flops / (us_layer * 1e-6) / 1e12, 2),
         "mfma_frac_of_fp8_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP8_TFLOPS, 4),
         "mfma_frac_of_mxfp4_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP4_TFLOPS, 4),
-        "block_rmsnorm_layer_hc_post": block, "unit_rows": unit_rows, "roofline": roofline, "cpu_baseline": cpu, "setup_s": round(t_setup, 1), "build_id": hip.build_id,
+        "block_rmsnorm_layer_hc_post": block, "checkpoint_load": load, "unit_rows": unit_rows, "roofline": roofline, "cpu_baseline": cpu, "setup_s": round(t_setup, 1), "build_id": hip.build_id,
     }
     if trace is not None:
         hip.graph_destroy(trace)

@@ -117,7 +117,7 @@ class Checkpoint:
             raise InvalidArg("validate_moe: bad argument")
         return [ln for ln in report.value.decode().split("\n") if ln]
 
-    def load_moe_layer(self, be: HipBackend, cfg: MoeConfig, prefix: str, naming: int, workers: int = 4,
+    def load_moe_layer(self, be: HipBackend, cfg: MoeConfig, prefix: str, naming: int, workers: int = 8,
                        pad_scale_rows: bool = False, hip_so: Optional[str] = None) -> Tuple[MoeLayer, LoadStats]:
         """Stream the layer into a packed device buffer; the returned layer holds `packed` and the routing bias
         only (no checkpoint-layout copy stays on the device)."""

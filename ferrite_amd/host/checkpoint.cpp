@@ -365,8 +365,54 @@ MoeCheckpointLoader::MoeCheckpointLoader(const std::string& so_path, int device)
 }
 
 MoeCheckpointLoader::~MoeCheckpointLoader() {
+    for (Slot& sl : slots_) release(sl);
     if (so_) dlclose(so_);
     delete api_;
+}
+
+void MoeCheckpointLoader::release(Slot& sl) {
+    if (sl.stream) { (void)hipStreamSynchronize(static_cast<hipStream_t>(sl.stream)); (void)hipStreamDestroy(static_cast<hipStream_t>(sl.stream)); }
+    for (void* ev : sl.done)
+        if (ev) (void)hipEventDestroy(static_cast<hipEvent_t>(ev));
+    if (sl.qdev) (void)hipFree(sl.qdev);
+    if (sl.dev) (void)hipFree(sl.dev);
+    if (sl.pinned) (void)hipHostFree(sl.pinned);
+    sl = Slot{};
+}
+
+// Staging resources live as long as the loader: a model has many layers and each load reuses them.
+void MoeCheckpointLoader::ensure_slots(int count, size_t bytes, size_t qbytes) const {
+    if ((int)slots_.size() < count) slots_.resize((size_t)count);
+    for (int i = 0; i < count; ++i) {
+        Slot& sl = slots_[(size_t)i];
+        if (!sl.stream) {
+            hipStream_t st = nullptr;
+            hipck(hipStreamCreateWithFlags(&st, hipStreamNonBlocking), "hipStreamCreate");   // default priority
+            sl.stream = st;
+        }
+        for (void*& ev : sl.done)
+            if (!ev) {
+                hipEvent_t e = nullptr;
+                hipck(hipEventCreateWithFlags(&e, hipEventDisableTiming), "hipEventCreate");
+                ev = e;
+            }
+        if (sl.bytes < bytes) {   // two halves of `bytes` each
+            if (sl.dev) (void)hipFree(sl.dev);
+            if (sl.pinned) (void)hipHostFree(sl.pinned);
+            sl.dev = sl.pinned = nullptr;
+            sl.bytes = 0;
+            hipck(hipHostMalloc(reinterpret_cast<void**>(&sl.pinned), 2 * bytes, hipHostMallocDefault), "hipHostMalloc");
+            hipck(hipMalloc(reinterpret_cast<void**>(&sl.dev), 2 * bytes), "hipMalloc");
+            sl.bytes = bytes;
+        }
+        if (sl.qbytes < qbytes) {
+            if (sl.qdev) (void)hipFree(sl.qdev);
+            sl.qdev = nullptr;
+            sl.qbytes = 0;
+            hipck(hipMalloc(reinterpret_cast<void**>(&sl.qdev), 2 * qbytes), "hipMalloc");
+            sl.qbytes = qbytes;
+        }
+    }
 }
 
 size_t MoeCheckpointLoader::packed_bytes(const ferrite_moe_shape& shape) const {
@@ -480,8 +526,9 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
 
     hipck(hipSetDevice(device_), "hipSetDevice");
 
-    // ---- router and bias: small, converted to f32 on the host when stored as bf16 ----
-    {
+    // ---- router and bias: small, converted to f32 on the host when stored as bf16; runs on the calling thread
+    //      while the workers stream the experts ----
+    auto load_router = [&]() {
         std::vector<float> rw(E * H), rb;
         auto to_f32 = [](const uint8_t* src, size_t es, size_t n, float* dst) {
             if (es == 4) { memcpy(dst, src, n * 4); return; }
@@ -502,8 +549,8 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
             to_f32(bias_src, bias_es, E, rb.data());
             hipck(hipMemcpy(router_bias_dev, rb.data(), E * 4, hipMemcpyHostToDevice), "hipMemcpy bias");
         }
-        hipck(hipDeviceSynchronize(), "hipDeviceSynchronize");
-    }
+        hipck(hipStreamSynchronize(nullptr), "hipStreamSynchronize");   // drw is freed on return
+    };
 
     // ---- experts: worker w stages experts w, w + W, ... through its own pinned buffer, device buffer and stream ----
     const int W = std::max(1, std::min(opt.workers, n_src));
@@ -511,32 +558,36 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
     std::atomic<bool> failed{false};
     std::mutex err_mu;
     std::string err;
+    size_t qbytes = 0;
+    if (!quantised) {
+        // room for the codes and scales the device quantiser writes (largest expert)
+        for (int e = 0; e < n_src; ++e) {
+            const size_t I = e == s.n_experts ? s.shared_inter : s.inter;
+            qbytes = std::max(qbytes, 3 * align256(I * H / 2) + 3 * align256(I * H / 32));
+        }
+    }
+    std::lock_guard<std::mutex> one_load_at_a_time(mu_);
+    ensure_slots(W, slot_bytes, qbytes);
     auto worker = [&](int wid) {
-        uint8_t* pinned = nullptr;
-        uint8_t* dev = nullptr;
-        uint8_t* qdev = nullptr;
-        hipStream_t st = nullptr;
+        const Slot& sl = slots_[(size_t)wid];
+        hipStream_t st = static_cast<hipStream_t>(sl.stream);
         try {
             hipck(hipSetDevice(device_), "hipSetDevice");
-            hipck(hipHostMalloc(reinterpret_cast<void**>(&pinned), slot_bytes, hipHostMallocDefault), "hipHostMalloc");
-            hipck(hipMalloc(reinterpret_cast<void**>(&dev), slot_bytes), "hipMalloc");
-            hipck(hipStreamCreateWithFlags(&st, hipStreamNonBlocking), "hipStreamCreate");
-            size_t qbytes = 0;
-            if (!quantised) {
-                // room for the codes and scales the device quantiser writes (largest expert)
-                for (int e = 0; e < n_src; ++e) {
-                    const size_t I = e == s.n_experts ? s.shared_inter : s.inter;
-                    qbytes = std::max(qbytes, 3 * align256(I * H / 2) + 3 * align256(I * H / 32));
-                }
-                hipck(hipMalloc(reinterpret_cast<void**>(&qdev), qbytes), "hipMalloc");
-            }
-            for (int e = wid; e < n_src && !failed.load(); e += W) {
+            int turn = 0;
+            for (int e = wid; e < n_src && !failed.load(); e += W, ++turn) {
+                // two halves per slot: the host fills one while the device copies and repacks the other
+                const int half = turn & 1;
+                uint8_t* pinned = sl.pinned + (size_t)half * sl.bytes;
+                uint8_t* dev = sl.dev + (size_t)half * sl.bytes;
+                uint8_t* qdev = sl.qdev ? sl.qdev + (size_t)half * sl.qbytes : nullptr;
+                hipEvent_t done = static_cast<hipEvent_t>(sl.done[half]);
                 const ExpertSrc& x = experts[e];
                 const size_t I = e == s.n_experts ? s.shared_inter : s.inter;
                 const size_t gu_pitch = quantised && opt.pad_scale_rows ? sf_plane_pitch(H / 32) : H / 32;
                 const size_t dn_pitch = quantised && opt.pad_scale_rows ? sf_plane_pitch(I / 32) : I / 32;
-                // the previous expert's pack kernels have read the device buffer, and its copy the pinned one
-                hipck(hipStreamSynchronize(st), "hipStreamSynchronize");
+                // the expert before the previous one used this half: its copy has read the pinned buffer and its
+                // pack kernels the device buffer
+                if (turn >= 2) hipck(hipEventSynchronize(done), "hipEventSynchronize");
                 size_t off = 0;
                 auto stage = [&](const uint8_t* src, size_t bytes) {
                     const size_t at = off;
@@ -582,6 +633,7 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
                 }
                 const int rc = api_->ferrite_moe_pack_expert(&s, e, &src, packed_dev, st);
                 if (rc) config_error(std::string("pack_expert: rc=") + std::to_string(rc) + " " + api_->ferrite_hip_last_error());
+                hipck(hipEventRecord(done, st), "hipEventRecord");
             }
             hipck(hipStreamSynchronize(st), "hipStreamSynchronize");
         } catch (const std::exception& ex) {
@@ -589,13 +641,17 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
             std::lock_guard<std::mutex> g(err_mu);
             if (err.empty()) err = ex.what();
         }
-        if (st) { (void)hipStreamSynchronize(st); (void)hipStreamDestroy(st); }
-        if (qdev) (void)hipFree(qdev);
-        if (dev) (void)hipFree(dev);
-        if (pinned) (void)hipHostFree(pinned);
+        (void)hipStreamSynchronize(st);   // also after a failure: nothing of this load is left in flight
     };
     std::vector<std::thread> threads;
     for (int w = 1; w < W; ++w) threads.emplace_back(worker, w);
+    try {
+        load_router();
+    } catch (const std::exception& ex) {
+        failed.store(true);
+        std::lock_guard<std::mutex> g(err_mu);
+        if (err.empty()) err = ex.what();
+    }
     worker(0);
     for (auto& t : threads) t.join();
     if (failed.load()) config_error(err);

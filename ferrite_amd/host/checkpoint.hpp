@@ -11,6 +11,7 @@
 #pragma once
 #include <cstddef>
 #include <cstdint>
+#include <mutex>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -88,7 +89,7 @@ struct LoadStats {
 };
 
 struct LoadOptions {
-    int workers = 4;             // staging threads, each with its own pinned buffer, device buffer and stream
+    int workers = 8;             // staging threads, each with its own pinned buffer, device buffer and stream
     bool pad_scale_rows = false; // stage scale planes with sf_plane_pitch rows (exercises the pitch argument)
 };
 
@@ -109,9 +110,21 @@ class MoeCheckpointLoader {
 
   private:
     struct Api;
+    struct Slot {              // one staging worker's resources; every buffer is two halves used in turn
+        uint8_t* pinned = nullptr;
+        uint8_t* dev = nullptr;
+        uint8_t* qdev = nullptr;   // output of the device quantiser (unquantised checkpoints only)
+        size_t bytes = 0, qbytes = 0;   // size of one half
+        void* stream = nullptr;
+        void* done[2] = {nullptr, nullptr};   // recorded after the pack kernels that read a half
+    };
+    void ensure_slots(int count, size_t bytes, size_t qbytes) const;
+    static void release(Slot& sl);
     Api* api_;
     void* so_ = nullptr;
     int device_ = 0;
+    mutable std::vector<Slot> slots_;
+    mutable std::mutex mu_;     // one load at a time per loader: the slots are shared state
 };
 
 }  // namespace ferrite

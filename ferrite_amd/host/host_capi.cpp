@@ -3,6 +3,7 @@
 #include <cstdio>
 #include <cstring>
 #include <memory>
+#include <string>
 
 #include "checkpoint.hpp"
 
@@ -11,6 +12,10 @@ using namespace ferrite;
 struct ferrite_ckpt {
     SafetensorsIndex index;
     std::unique_ptr<MappedFile> file;
+    // the loader (library handle, staging buffers, streams) is kept between layers of the same shard
+    std::unique_ptr<MoeCheckpointLoader> loader;
+    std::string loader_so;
+    int loader_device = -1;
 };
 
 static void set_err(char* err, size_t errlen, const char* msg) {
@@ -69,7 +74,13 @@ extern "C" int ferrite_ckpt_load_moe_layer(const ferrite_ckpt* ck, const char* h
     try {
         if (!ck || !hip_so_path || !prefix || !shape || naming < 0 || naming > 1)
             throw FerriteError(FerriteError::InvalidArg, "null or out-of-range argument");
-        MoeCheckpointLoader loader(hip_so_path, device);
+        ferrite_ckpt* mck = const_cast<ferrite_ckpt*>(ck);
+        if (!mck->loader || mck->loader_so != hip_so_path || mck->loader_device != device) {
+            mck->loader.reset(new MoeCheckpointLoader(hip_so_path, device));
+            mck->loader_so = hip_so_path;
+            mck->loader_device = device;
+        }
+        const MoeCheckpointLoader& loader = *mck->loader;
         LoadOptions opt;
         if (workers > 0) opt.workers = workers;
         opt.pad_scale_rows = pad_scale_rows != 0;
