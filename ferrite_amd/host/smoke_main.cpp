@@ -9,6 +9,7 @@
 #include <numeric>
 
 #include "hip_backend.hpp"
+#include "checkpoint.hpp"
 
 using namespace ferrite;
 
@@ -220,6 +221,100 @@ static void graph_capture_smoke(HipBackend& b) {   // gpu_smoke.rs:268-306: capt
     b.graph_destroy(trace);
 }
 
+// A shard written here (safetensors: 8-byte header length, JSON header, tensors back to back) is streamed by the
+// checkpoint loader into a packed buffer that must equal, byte for byte, the one load_moe_layer builds from the
+// same tensors in memory (the names are those of crates/ferrite-models/src/dsv41/weights.rs:333-341).
+static void checkpoint_loader_roundtrip(HipBackend& b, const std::string& so_path) {
+    const size_t H = 256, I = 128, Is = 128, E = 3;
+    ferrite_moe_shape shape{(int)H, (int)E, 2, (int)I, (int)Is, 1, 1, 1.0f, 7.0f};
+    uint32_t rng = 12345u;
+    auto fill = [&](std::vector<uint8_t>& v, size_t n, bool scale) {
+        v.resize(n);
+        for (auto& x : v) { rng = rng * 1664525u + 1013904223u; x = scale ? (uint8_t)(118 + (rng >> 28)) : (uint8_t)(rng >> 24); }
+    };
+    std::vector<float> router(E * H), bias(E);
+    for (size_t i = 0; i < E * H; ++i) router[i] = bex(i, 3);
+    for (size_t i = 0; i < E; ++i) bias[i] = bex(i, 1);
+    std::vector<uint8_t> gw, gs, uw, us, dw, ds, sgw, sgs, suw, sus, sdw, sds;
+    fill(gw, E * I * H / 2, false); fill(gs, E * I * H / 32, true); fill(uw, E * I * H / 2, false); fill(us, E * I * H / 32, true);
+    fill(dw, E * H * I / 2, false); fill(ds, E * H * I / 32, true);
+    fill(sgw, Is * H / 2, false); fill(sgs, Is * H / 32, true); fill(suw, Is * H / 2, false); fill(sus, Is * H / 32, true);
+    fill(sdw, H * Is / 2, false); fill(sds, H * Is / 32, true);
+    MoeHostWeights hw{router.data(), bias.data(), gw.data(), gs.data(), uw.data(), us.data(), dw.data(), ds.data(),
+                      sgw.data(), sgs.data(), suw.data(), sus.data(), sdw.data(), sds.data()};
+    MoeLayerDev mem = b.load_moe_layer(shape, hw);
+
+    std::string header = "{";
+    std::string blob;
+    auto add = [&](const std::string& name, const char* dtype, size_t r, size_t c, const void* data, size_t bytes) {
+        if (header.size() > 1) header += ",";
+        header += "\"" + name + "\":{\"dtype\":\"" + dtype + "\",\"shape\":[" + std::to_string(r) +
+                  (c ? "," + std::to_string(c) : std::string()) + "],\"data_offsets\":[" + std::to_string(blob.size()) + "," +
+                  std::to_string(blob.size() + bytes) + "]}";
+        blob.append(static_cast<const char*>(data), bytes);
+    };
+    const std::string p = "layers.6.ffn";
+    add(p + ".gate.weight", "F32", E, H, router.data(), E * H * 4);
+    add(p + ".gate.bias", "F32", E, 0, bias.data(), E * 4);
+    for (size_t e = 0; e <= E; ++e) {
+        const bool sh = e == E;
+        const std::string q = sh ? p + ".shared_experts" : p + ".experts." + std::to_string(e);
+        const size_t inter = sh ? Is : I;
+        const size_t cw = inter * H / 2, cs = inter * H / 32;
+        add(q + ".w1.weight", "I8", inter, H / 2, (sh ? sgw.data() : gw.data() + e * cw), cw);
+        add(q + ".w1.scale", "F8_E8M0", inter, H / 32, (sh ? sgs.data() : gs.data() + e * cs), cs);
+        add(q + ".w2.weight", "I8", H, inter / 2, (sh ? sdw.data() : dw.data() + e * cw), cw);
+        add(q + ".w2.scale", "F8_E8M0", H, inter / 32, (sh ? sds.data() : ds.data() + e * cs), cs);
+        add(q + ".w3.weight", "I8", inter, H / 2, (sh ? suw.data() : uw.data() + e * cw), cw);
+        add(q + ".w3.scale", "F8_E8M0", inter, H / 32, (sh ? sus.data() : us.data() + e * cs), cs);
+    }
+    header += "}";
+    while (header.size() % 8) header += ' ';
+    char path[] = "/tmp/ferrite_smoke_XXXXXX";
+    const int fd = mkstemp(path);
+    CHECK(fd >= 0, "mkstemp failed");
+    if (fd < 0) return;
+    FILE* f = fdopen(fd, "wb");
+    const uint64_t hlen = header.size();
+    fwrite(&hlen, 8, 1, f);
+    fwrite(header.data(), 1, header.size(), f);
+    fwrite(blob.data(), 1, blob.size(), f);
+    fclose(f);
+
+    SafetensorsIndex index = SafetensorsIndex::read_header(path);
+    const auto missing = index.validate(moe_layer_specs(MoeNaming::Dsv41, p, shape));
+    CHECK(missing.empty(), "validate reports %zu missing tensors (first: %s)", missing.size(), missing.empty() ? "" : missing[0].c_str());
+    CHECK(index.tensors.size() == 2 + 6 * (E + 1), "index holds %zu tensors", index.tensors.size());
+    MappedFile file(path);
+    MoeCheckpointLoader loader(so_path, 0);
+    const size_t pb = loader.packed_bytes(shape);
+    CHECK(pb == mem.packed.bytes, "packed size %zu vs %zu", pb, mem.packed.bytes);
+    DevBuf packed(pb), dbias(E * 4);
+    LoadOptions opt;
+    opt.workers = 3;
+    opt.pad_scale_rows = true;
+    const LoadStats st = loader.load_layer(file, index, MoeNaming::Dsv41, p, shape, static_cast<uint8_t*>(packed.ptr),
+                                           static_cast<float*>(dbias.ptr), opt);
+    std::vector<uint8_t> a(pb), c(pb);
+    packed.download(a.data(), pb);
+    mem.packed.download(c.data(), pb);
+    CHECK(std::memcmp(a.data(), c.data(), pb) == 0, "packed buffer from the shard differs from the memory-loaded one");
+    std::vector<float> hb(E);
+    dbias.download(hb.data(), E * 4);
+    CHECK(std::memcmp(hb.data(), bias.data(), E * 4) == 0, "routing bias differs");
+    bool threw = false;
+    try {
+        loader.load_layer(file, index, MoeNaming::Dsv41, "layers.7.ffn", shape, static_cast<uint8_t*>(packed.ptr),
+                          static_cast<float*>(dbias.ptr), opt);
+    } catch (const FerriteError& e) {
+        threw = std::string(e.what()).find("missing tensor layers.7.ffn.gate.weight") != std::string::npos;
+    }
+    CHECK(threw, "a missing layer must be reported by name");
+    std::remove(path);
+    std::printf("[checkpoint] %llu source bytes -> %llu packed, %d workers\n", (unsigned long long)st.source_bytes,
+                (unsigned long long)st.packed_bytes, st.workers);
+}
+
 int main(int argc, char** argv) {
     if (argc < 2) { std::printf("usage: %s libferrite_hip.so\n", argv[0]); return 2; }
     try {
@@ -231,7 +326,8 @@ int main(int argc, char** argv) {
         hc_post_vs_host_loop(b); std::printf("hc_post ok\n"); std::fflush(stdout);
         moe_route_noaux_tc(b); std::printf("moe_route ok\n"); std::fflush(stdout);
         moe_fused_parity(b); std::fflush(stdout);
-        graph_capture_smoke(b); std::printf("graph ok\n");
+        graph_capture_smoke(b); std::printf("graph ok\n"); std::fflush(stdout);
+        checkpoint_loader_roundtrip(b, argv[1]); std::printf("checkpoint ok\n");
     } catch (const std::exception& e) {
         std::printf("EXCEPTION: %s\n", e.what());
         return 1;
