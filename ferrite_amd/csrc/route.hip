@@ -555,36 +555,41 @@ struct HeadArgs {
     PermArgs perm;
 };
 
-// T = tokens per block (1, or 2 when one token per block would need more than one round of blocks on the chip).
-template <int T>
+// T = tokens per block, W = product groups (of four k, all tokens together) per ring buffer.
+//   up to 256 blocks (one per CU)  : T 1, W 32 - 64 KiB of ring, the fewest barriers per chain
+//   up to 512 blocks               : T 1, W 16 - 32 KiB of ring and under 128 registers, so two blocks share a CU and
+//                                    their chain waves run side by side (192 tokens x 2 expert blocks: 44.7 us
+//                                    against 60.6 us for two interleaved chains per block)
+//   more                           : T 2, W 32 - two interleaved chains per block, the weights fetched once
+template <int T, int W>
 struct HeadCfg {
-    static constexpr int CH = 32 / T;                        // groups of four k per chunk
+    static constexpr int CH = W / T;                         // groups of four k per chunk and token
     static constexpr int PW = (CH + HD_NP - 1) / HD_NP;      // groups per producer wave and chunk
-    static constexpr size_t RING_BYTES = 2 * (size_t)CH * T * 1024;   // 64 KiB
+    static constexpr size_t RING_BYTES = 2 * (size_t)W * 1024;
 };
 
-template <int T>
+template <int T, int W>
 struct HeadSet {
-    float4 w[HeadCfg<T>::PW];
+    float4 w[HeadCfg<T, W>::PW];
 };
 
 // Producer P (0..HD_NP-1) owns groups P, P+HD_NP, ... of every chunk.  Chunks past the end re-read the last one
 // (never consumed), which keeps every load unconditional.
-template <int T, int P>
-__device__ __forceinline__ void head_pload(HeadSet<T>& st, const float4* __restrict__ wp, int Epad, int c, int nch) {
-    constexpr int CH = HeadCfg<T>::CH;
+template <int T, int W, int P>
+__device__ __forceinline__ void head_pload(HeadSet<T, W>& st, const float4* __restrict__ wp, int Epad, int c, int nch) {
+    constexpr int CH = HeadCfg<T, W>::CH;
     const float4* base = wp + (size_t)min(c, nch - 1) * CH * Epad;
 #pragma unroll
-    for (int i = 0; i < HeadCfg<T>::PW; ++i)
+    for (int i = 0; i < HeadCfg<T, W>::PW; ++i)
         if (P + HD_NP * i < CH) st.w[i] = base[(size_t)(P + HD_NP * i) * Epad];
 }
 
 // products of the chunk's group j for token ti go to slot (j*T + ti)*64 + lane of the ring buffer
-template <int T, int P>
-__device__ __forceinline__ void head_pmul(const HeadSet<T>& st, const float4* xl, int nk4, int c, float4* buf, int lane) {
-    constexpr int CH = HeadCfg<T>::CH;
+template <int T, int W, int P>
+__device__ __forceinline__ void head_pmul(const HeadSet<T, W>& st, const float4* xl, int nk4, int c, float4* buf, int lane) {
+    constexpr int CH = HeadCfg<T, W>::CH;
 #pragma unroll
-    for (int i = 0; i < HeadCfg<T>::PW; ++i) {
+    for (int i = 0; i < HeadCfg<T, W>::PW; ++i) {
         const int j = P + HD_NP * i;
         if (j < CH) {
             const float4 wv = st.w[i];
@@ -600,34 +605,34 @@ __device__ __forceinline__ void head_pmul(const HeadSet<T>& st, const float4* xl
 
 // Products of chunk c+1 are made while the chain consumes chunk c; register set c%4 holds the weights of chunk c
 // and is reloaded for chunk c+4 as soon as it has been used.
-template <int T, int P>
+template <int T, int W, int P>
 __device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int Epad, int nk4, const float4* xl,
                                               float4* ring, int lane) {
-    constexpr int CH = HeadCfg<T>::CH;
+    constexpr int CH = HeadCfg<T, W>::CH;
     const int nch = nk4 / CH;
     float4* b0 = ring;
     float4* b1 = ring + CH * T * 64;
-    HeadSet<T> s0, s1, s2, s3;
-    head_pload<T, P>(s0, wp, Epad, 0, nch);
-    head_pload<T, P>(s1, wp, Epad, 1, nch);
-    head_pload<T, P>(s2, wp, Epad, 2, nch);
-    head_pload<T, P>(s3, wp, Epad, 3, nch);
+    HeadSet<T, W> s0, s1, s2, s3;
+    head_pload<T, W, P>(s0, wp, Epad, 0, nch);
+    head_pload<T, W, P>(s1, wp, Epad, 1, nch);
+    head_pload<T, W, P>(s2, wp, Epad, 2, nch);
+    head_pload<T, W, P>(s3, wp, Epad, 3, nch);
     __syncthreads();   // x is in LDS
-    head_pmul<T, P>(s0, xl, nk4, 0, b0, lane);
-    head_pload<T, P>(s0, wp, Epad, 4, nch);
+    head_pmul<T, W, P>(s0, xl, nk4, 0, b0, lane);
+    head_pload<T, W, P>(s0, wp, Epad, 4, nch);
     __syncthreads();
     for (int c = 0; c < nch; c += 4) {
-        head_pmul<T, P>(s1, xl, nk4, min(c + 1, nch - 1), b1, lane);
-        head_pload<T, P>(s1, wp, Epad, c + 5, nch);
+        head_pmul<T, W, P>(s1, xl, nk4, min(c + 1, nch - 1), b1, lane);
+        head_pload<T, W, P>(s1, wp, Epad, c + 5, nch);
         __syncthreads();
-        head_pmul<T, P>(s2, xl, nk4, min(c + 2, nch - 1), b0, lane);
-        head_pload<T, P>(s2, wp, Epad, c + 6, nch);
+        head_pmul<T, W, P>(s2, xl, nk4, min(c + 2, nch - 1), b0, lane);
+        head_pload<T, W, P>(s2, wp, Epad, c + 6, nch);
         __syncthreads();
-        head_pmul<T, P>(s3, xl, nk4, min(c + 3, nch - 1), b1, lane);
-        head_pload<T, P>(s3, wp, Epad, c + 7, nch);
+        head_pmul<T, W, P>(s3, xl, nk4, min(c + 3, nch - 1), b1, lane);
+        head_pload<T, W, P>(s3, wp, Epad, c + 7, nch);
         __syncthreads();
-        head_pmul<T, P>(s0, xl, nk4, min(c + 4, nch - 1), b0, lane);
-        head_pload<T, P>(s0, wp, Epad, c + 8, nch);
+        head_pmul<T, W, P>(s0, xl, nk4, min(c + 4, nch - 1), b0, lane);
+        head_pload<T, W, P>(s0, wp, Epad, c + 8, nch);
         __syncthreads();
     }
 }
@@ -635,9 +640,9 @@ __device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int
 // The chains over one chunk of products: batches of eight LDS reads (8/T groups of four k for each of the T
 // tokens), one wait per batch (0xC87F: lgkmcnt <= 8, i.e. everything but the batch just issued; 0xC07F: lgkmcnt 0),
 // 32 adds per batch, dependent within a token's chain.
-template <int T>
+template <int T, int W>
 __device__ __forceinline__ void head_consume(float (&s)[T], const float4* buf, int lane) {
-    constexpr int NB = HeadCfg<T>::CH * T / 8;   // batches per chunk (4)
+    constexpr int NB = HeadCfg<T, W>::CH * T / 8;   // batches per chunk (4)
     float4 r[2][8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) r[0][j] = buf[j * 64 + lane];
@@ -667,27 +672,27 @@ __device__ __forceinline__ void head_consume(float (&s)[T], const float4* buf, i
 }
 
 // Barriers pair one to one with head_producer's.
-template <int T>
+template <int T, int W>
 __device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const float4* ring, int lane) {
-    constexpr int CH = HeadCfg<T>::CH;
+    constexpr int CH = HeadCfg<T, W>::CH;
     const int nch = nk4 / CH;
     const float4* b0 = ring;
     const float4* b1 = ring + CH * T * 64;
     __syncthreads();
     __syncthreads();
     for (int c = 0; c < nch; c += 4) {
-        head_consume<T>(s, b0, lane);
+        head_consume<T, W>(s, b0, lane);
         __syncthreads();
-        if (c + 1 < nch) head_consume<T>(s, b1, lane);
+        if (c + 1 < nch) head_consume<T, W>(s, b1, lane);
         __syncthreads();
-        if (c + 2 < nch) head_consume<T>(s, b0, lane);
+        if (c + 2 < nch) head_consume<T, W>(s, b0, lane);
         __syncthreads();
-        if (c + 3 < nch) head_consume<T>(s, b1, lane);
+        if (c + 3 < nch) head_consume<T, W>(s, b1, lane);
         __syncthreads();
     }
 }
 
-template <typename XT, bool kFused, int T>
+template <typename XT, bool kFused, int T, int W>
 __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
     extern __shared__ __align__(16) unsigned char head_lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -707,7 +712,7 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
         return;
     }
     float4* ring = reinterpret_cast<float4*>(head_lds);
-    float4* xl = reinterpret_cast<float4*>(head_lds + HeadCfg<T>::RING_BYTES);   // [T][H/4]
+    float4* xl = reinterpret_cast<float4*>(head_lds + HeadCfg<T, W>::RING_BYTES);   // [T][H/4]
     const int nk4 = H / 4;   // a multiple of 32 (H % 128 == 0)
     const float4* wp = reinterpret_cast<const float4*>(a.wt) + (size_t)eb * 64 + lane;
     for (int i = tid; i < T * nk4; i += 512) {
@@ -727,13 +732,13 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
 #pragma unroll
     for (int ti = 0; ti < T; ++ti) s[ti] = 0.0f;
     switch (wave) {
-        case 0: head_consumer<T>(s, nk4, ring, lane); break;
-        case 1: head_producer<T, 0>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 2: head_producer<T, 1>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 3: head_producer<T, 2>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 5: head_producer<T, 3>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 6: head_producer<T, 4>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 7: head_producer<T, 5>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 0: head_consumer<T, W>(s, nk4, ring, lane); break;
+        case 1: head_producer<T, W, 0>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 2: head_producer<T, W, 1>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 3: head_producer<T, W, 2>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 5: head_producer<T, W, 3>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 6: head_producer<T, W, 4>(wp, a.Epad, nk4, xl, ring, lane); break;
+        case 7: head_producer<T, W, 5>(wp, a.Epad, nk4, xl, ring, lane); break;
         default: __syncthreads(); break;   // its share of x is in LDS before it goes
     }
     if (wave != 0) return;   // from here on the block is wave 0 alone; LDS is free for the scratch below
@@ -770,11 +775,18 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
 }
 
 // tokens per block: two when one per block would not fit the chip's 256 CUs in one round
-static int head_tokens_per_block(int n, int eblocks) { return (long)n * eblocks > 256 ? 2 : 1; }
+// (tokens per block, ring width) for n tokens x eblocks blocks of 64 experts: see HeadCfg.
+struct HeadShape { int T, W; };
+static HeadShape head_shape(int n, int eblocks) {
+    const long blocks = (long)n * eblocks;
+    if (blocks <= 256) return {1, 32};
+    if (blocks <= 512) return {1, 16};
+    return {2, 32};
+}
 
 static size_t head_lds_bytes(int n, int H, int E, bool fused) {
-    const int T = head_tokens_per_block(n, (E + 63) / 64);
-    size_t b = 64 * 1024 + (size_t)T * H * 4;
+    const HeadShape hs = head_shape(n, (E + 63) / 64);
+    size_t b = 2 * (size_t)hs.W * 1024 + (size_t)hs.T * H * 4;
     if (fused) {
         if (b < sizeof(RouteScratch)) b = sizeof(RouteScratch);
         size_t p = perm_block_lds_bytes(n, E);
@@ -787,20 +799,22 @@ bool head_supported(int n, int H, int E) {
     return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, H, E, true) <= 160 * 1024;
 }
 
-template <typename XT, bool kFused, int T>
+template <typename XT, bool kFused, int T, int W>
 static int launch_head_tt(const HeadArgs& a, int quant, size_t lds, hipStream_t st) {
     static size_t raised = 0;
-    int rc = set_lds_limit(moe_head_kernel<XT, kFused, T>, lds, &raised);
+    int rc = set_lds_limit(moe_head_kernel<XT, kFused, T, W>, lds, &raised);
     if (rc) return rc;
     dim3 grid(a.Epad / 64 + quant, (a.n + T - 1) / T);
-    moe_head_kernel<XT, kFused, T><<<grid, 512, lds, st>>>(a);
+    moe_head_kernel<XT, kFused, T, W><<<grid, 512, lds, st>>>(a);
     return check_launch("moe_head");
 }
 
 template <typename XT, bool kFused>
 static int launch_head_t(const HeadArgs& a, int quant, size_t lds, hipStream_t st) {
-    if (head_tokens_per_block(a.n, a.Epad / 64) == 2) return launch_head_tt<XT, kFused, 2>(a, quant, lds, st);
-    return launch_head_tt<XT, kFused, 1>(a, quant, lds, st);
+    const HeadShape hs = head_shape(a.n, a.Epad / 64);
+    if (hs.T == 2) return launch_head_tt<XT, kFused, 2, 32>(a, quant, lds, st);
+    if (hs.W == 16) return launch_head_tt<XT, kFused, 1, 16>(a, quant, lds, st);
+    return launch_head_tt<XT, kFused, 1, 32>(a, quant, lds, st);
 }
 
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,

@@ -177,6 +177,21 @@ def test_layer_unfused_head_path(hip, oracle):
     assert max_abs_rel(out, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
 
 
+@pytest.mark.parametrize("n,e,bf16", [(100, 128, False), (200, 128, True), (200, 192, False), (256, 320, True), (65, 64, False)])
+def test_layer_fused_head_shapes(hip, oracle, n, e, bf16):
+    """The fused routing kernel picks its block shape from n x (blocks of 64 experts): one token per block with a
+    wide product ring (up to 256 blocks), one token with a narrow ring so that two blocks share a CU (up to 512),
+    two tokens per block beyond that.  Logits, routing and tables are bit-exact in each, for f32 and bf16 input,
+    with n odd against the two-token blocks and the separate permutation launch (n > 64)."""
+    cfg = synth.MoeConfig(n, 384, e, 4, 128, 128, 4, 2, act_bf16=bf16)
+    inp = synth.make_inputs(cfg, seed=23)
+    layer = hip.load_moe_layer(inp)
+    ref = oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)
+    out, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8, bf16=bf16)
+    check_routing(v, ref, oracle, cfg)
+    assert max_abs_rel(out, ref["out"]) <= TOL_MFMA
+
+
 @pytest.mark.parametrize("n", [40, 700])
 def test_layer_all_tokens_on_the_same_experts(hip, oracle, n):
     """Maximum skew: a bias of +50 on three experts of one group makes every token pick exactly those (the sigmoid
