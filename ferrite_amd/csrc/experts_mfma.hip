@@ -121,27 +121,37 @@ struct StreamRegs {
     u4v sc[2];
 };
 
+// kKeep: plain loads, whose lines stay in the XCD's L2 for the other units of the same expert that follow this
+// block; otherwise non-temporal loads, which stream about 10 % faster but are not retained.
+template <bool kKeep>
+__device__ __forceinline__ u4v stream_ld(const u4v* p) {
+    if constexpr (kKeep) return *p;
+    else return __builtin_nontemporal_load(p);
+}
+
+template <bool kKeep>
 __device__ __forceinline__ void stream_load_group(StreamRegs& r, const u4v* __restrict__ wp,
                                                   const u4v* __restrict__ sp, int KT, int lane, int g4, int buf) {
-    r.sc[buf] = __builtin_nontemporal_load(&sp[(size_t)g4 * 64 + lane]);
+    r.sc[buf] = stream_ld<kKeep>(&sp[(size_t)g4 * 64 + lane]);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
         const int kt = g4 * 4 + q;
         if (kt < KT) {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                r.a[buf][q][t] = __builtin_nontemporal_load(&wp[((size_t)kt * 4 + t) * 64 + lane]);
+                r.a[buf][q][t] = stream_ld<kKeep>(&wp[((size_t)kt * 4 + t) * 64 + lane]);
         }
     }
 }
 
 // The item's group 0 must already be in flight in buffer 0 (stream_load_group(..., 0, 0)): callers issue it
 // before they fill LDS, so the first weights travel while the activations are staged.
+template <bool kKeep>
 __device__ __forceinline__ void stream_item(StreamRegs& r, const u4v* __restrict__ wp, const u4v* __restrict__ sp,
                                             int KT, const u4v* bq, const uint32_t* bsc, int lane, v4f (&acc)[4]) {
     const int KT4 = (KT + 3) >> 2;
     for (int g4 = 0; g4 < KT4; g4 += 2) {
-        if (g4 + 1 < KT4) stream_load_group(r, wp, sp, KT, lane, g4 + 1, 1);
+        if (g4 + 1 < KT4) stream_load_group<kKeep>(r, wp, sp, KT, lane, g4 + 1, 1);
         {
             const uint32_t bs = bsc[g4 * 64 + lane];
             const int kt = g4 * 4;
@@ -151,7 +161,7 @@ __device__ __forceinline__ void stream_item(StreamRegs& r, const u4v* __restrict
             if (kt + 3 < KT) mfma_step<3>(r.a[0][3], r.sc[0], bq, bs, kt + 3, lane, acc);
         }
         if (g4 + 1 < KT4) {
-            if (g4 + 2 < KT4) stream_load_group(r, wp, sp, KT, lane, g4 + 2, 0);
+            if (g4 + 2 < KT4) stream_load_group<kKeep>(r, wp, sp, KT, lane, g4 + 2, 0);
             const uint32_t bs = bsc[(g4 + 1) * 64 + lane];
             const int kt = (g4 + 1) * 4;
             mfma_step<0>(r.a[1][0], r.sc[1], bq, bs, kt, lane, acc);
@@ -209,23 +219,43 @@ __device__ __forceinline__ bool unit_ok(const MfmaArgs& a, int e, int row0, int 
     return e >= 0 && e < a.n_experts && row0 + nrows <= nk;
 }
 
+// Block -> (unit, item group).  Hardware deals consecutive blocks round-robin over the 8 XCDs; the live work
+// (n_units * groups) is cut into 8 contiguous ranges, one per XCD, so that the blocks of one expert share an L2.
+// Within a range the order is (expert, item group, unit of the expert): the units of an expert that need the
+// same weight tiles are dispatched back to back, run in lockstep and fetch those tiles from HBM once (with the
+// units of an expert a whole item-group sweep apart, or on different XCDs, each of them fetched them again).
+// Used by the 128-row kernels (2-3 units per expert) and by the 16-row kernels (the shared expert's n/16 units, an
+// expert with more than 16 rows).  Returns false for blocks without work or with inconsistent tables.
+__device__ __forceinline__ bool unit_block_work(const MfmaArgs& a, int groups, int& u, int& ig, int& ne) {
+    const int n_units = min(*a.n_units, a.max_units);
+    const int total = n_units * groups, per_xcd = (total + 7) >> 3;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int v = xcd * per_xcd + slot;
+    if (slot >= per_xcd || v >= total) return false;
+    const int up = v / groups;                       // some unit of the expert whose segment holds v
+    const int first = a.unit_first[up];
+    ne = a.unit_count[up];
+    if (first < 0 || ne < 1 || up < first || up >= first + ne || first + ne > n_units) return false;
+    const int vl = v - first * groups;               // 0 .. ne * groups - 1
+    ig = vl / ne;
+    u = first + (vl - ig * ne);
+    return true;
+}
+
 // gate/up GEMM + clamped SwiGLU + e4m3-per-32 quantisation of the result.
-// grid (ceil(items / WAVES), max_units); wave w of block b owns item b*WAVES + w of the unit's expert.
-template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, const uint8_t* __restrict__ xq,
-                                                                  const uint8_t* __restrict__ xs,
-                                                                  const int32_t* __restrict__ gather_src,
-                                                                  uint8_t* __restrict__ act_q,
-                                                                  uint8_t* __restrict__ act_s) {
-    extern __shared__ __align__(16) unsigned char lds_raw[];
-    const int u = blockIdx.y;
-    if (u >= *a.n_units) return;
+// grid: unit_block_work over groups = ceil(items / WAVES) item groups; wave w of item group ig owns item
+// ig*WAVES + w of the unit's expert.
+template <int WAVES, bool kKeep>
+__device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, const uint8_t* __restrict__ xq,
+                                             const uint8_t* __restrict__ xs, const int32_t* __restrict__ gather_src,
+                                             uint8_t* __restrict__ act_q, uint8_t* __restrict__ act_s,
+                                             unsigned char* lds_raw) {
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;   // tables from an uninitialised workspace must not cause a fault
     const bool shared = e == a.n_experts;
     const int inter = shared ? a.shared_inter : a.inter;
     const int items = inter / 32;
-    if ((int)blockIdx.x * WAVES >= items) return;
+    if (ig * WAVES >= items) return;
     const int H = a.hidden, KT = H / 128, KT4 = (KT + 3) / 4;
     u4v* bq = reinterpret_cast<u4v*>(lds_raw);
     uint32_t* bsc = reinterpret_cast<uint32_t*>(lds_raw + (size_t)H * 16);
@@ -237,21 +267,21 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
         return (i < 0 || i >= nk) ? -1 : i / topk;
     };
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int item = blockIdx.x * WAVES + wave;
+    const int item = ig * WAVES + wave;
     const bool live = item < items;
     const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
     const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
     const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
     const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
     StreamRegs regs;
-    if (live) stream_load_group(regs, wp, sp, KT, lane, 0, 0);   // weights fly while the activations are staged
+    if (live) stream_load_group<kKeep>(regs, wp, sp, KT, lane, 0, 0);   // weights fly while the activations are staged
     fill_b_operand(xq, xs, H, nrows, row_src, bq, bsc);
     __syncthreads();
     if (!live) return;
     v4f acc[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-    stream_item(regs, wp, sp, KT, bq, bsc, lane, acc);
+    stream_item<kKeep>(regs, wp, sp, KT, bq, bsc, lane, acc);
 
     // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
     float r0[4], r1[4];
@@ -277,14 +307,26 @@ __global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, co
     }
 }
 
-// down GEMM: y[row][h] for the unit's rows.  grid (ceil(items / (WAVES*IPW)), max_units); item = 64 rows of H.
-template <int WAVES, int IPW>
-__global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const uint8_t* __restrict__ act_q,
-                                                               const uint8_t* __restrict__ act_s,
-                                                               float* __restrict__ y) {
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
+                                                                  const uint8_t* __restrict__ xs,
+                                                                  const int32_t* __restrict__ gather_src,
+                                                                  uint8_t* __restrict__ act_q,
+                                                                  uint8_t* __restrict__ act_s) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    const int u = blockIdx.y;
-    if (u >= *a.n_units) return;
+    int u, ig, ne;
+    if (!unit_block_work(a, groups, u, ig, ne)) return;
+    // an expert with several units: its weights are wanted again by the blocks that follow on this XCD
+    if (ne > 1) gate_up_unit<WAVES, true>(a, u, ig, xq, xs, gather_src, act_q, act_s, lds_raw);
+    else gate_up_unit<WAVES, false>(a, u, ig, xq, xs, gather_src, act_q, act_s, lds_raw);
+}
+
+// down GEMM: y[row][h] for the unit's rows.  grid: unit_block_work over groups = ceil(items / (WAVES*IPW)); item =
+// 64 rows of H.
+template <int WAVES, int IPW, bool kKeep>
+__device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, const uint8_t* __restrict__ act_q,
+                                          const uint8_t* __restrict__ act_s, float* __restrict__ y,
+                                          unsigned char* lds_raw) {
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
@@ -294,12 +336,12 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
     u4v* bq = reinterpret_cast<u4v*>(lds_raw);
     uint32_t* bsc = reinterpret_cast<uint32_t*>(lds_raw + (size_t)a.act_ld * 16);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int item0 = (blockIdx.x * WAVES + wave) * IPW;
+    const int item0 = (ig * WAVES + wave) * IPW;
     StreamRegs regs;
     if (item0 < items) {   // the first item's weights fly while the activations are staged
         const uint8_t* cb = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
         const uint8_t* sb = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
-        stream_load_group(regs, reinterpret_cast<const u4v*>(cb) + (size_t)item0 * KT * 256,
+        stream_load_group<kKeep>(regs, reinterpret_cast<const u4v*>(cb) + (size_t)item0 * KT * 256,
                           reinterpret_cast<const u4v*>(sb) + (size_t)item0 * KT4 * 64, KT, lane, 0, 0);
     }
     // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
@@ -329,11 +371,11 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
         if (item >= items) break;
         const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
         const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
-        if (ii > 0) stream_load_group(regs, wp, sp, KT, lane, 0, 0);
+        if (ii > 0) stream_load_group<kKeep>(regs, wp, sp, KT, lane, 0, 0);
         v4f acc[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-        stream_item(regs, wp, sp, KT, bq, bsc, lane, acc);
+        stream_item<kKeep>(regs, wp, sp, KT, bq, bsc, lane, acc);
         if (c < nrows) {
             float* dst = y + (size_t)(row0 + c) * H + (size_t)item * 64 + g * 4;
 #pragma unroll
@@ -341,6 +383,17 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, const
                 *reinterpret_cast<float4*>(dst + t * 16) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
         }
     }
+}
+
+template <int WAVES, int IPW>
+__global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
+                                                               const uint8_t* __restrict__ act_s,
+                                                               float* __restrict__ y) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int u, ig, ne;
+    if (!unit_block_work(a, groups, u, ig, ne)) return;
+    if (ne > 1) down_unit<WAVES, IPW, true>(a, u, ig, act_q, act_s, y, lds_raw);
+    else down_unit<WAVES, IPW, false>(a, u, ig, act_q, act_s, y, lds_raw);
 }
 
 
@@ -472,27 +525,6 @@ __device__ __forceinline__ void pf_mainloop(const PfCtx& c, u4v* lds, v4f (&acc)
     if (rem > 2) pf_step<2>(c, lds, kt + 2, asc, bsc, acc);
 }
 
-// Block -> (unit, item group).  Hardware deals consecutive blocks round-robin over the 8 XCDs; the live work
-// (n_units * groups) is cut into 8 contiguous ranges, one per XCD, so that the blocks of one expert share an L2.
-// Within a range the order is (expert, item group, unit of the expert): the 2-3 units of an expert that need the
-// same weight tiles are dispatched back to back, run in lockstep and fetch those tiles from HBM once (with the
-// units of an expert a whole item-group sweep apart, the second one found them evicted and HBM traffic doubled,
-// which is what bounded the kernel).  Returns false for blocks without work or with inconsistent tables.
-__device__ __forceinline__ bool pf_block_work(const MfmaArgs& a, int groups, int& u, int& ig) {
-    const int n_units = min(*a.n_units, a.max_units);
-    const int total = n_units * groups, per_xcd = (total + 7) >> 3;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int v = xcd * per_xcd + slot;
-    if (slot >= per_xcd || v >= total) return false;
-    const int up = v / groups;                       // some unit of the expert whose segment holds v
-    const int first = a.unit_first[up], ne = a.unit_count[up];
-    if (first < 0 || ne < 1 || up < first || up >= first + ne || first + ne > n_units) return false;
-    const int vl = v - first * groups;               // 0 .. ne * groups - 1
-    ig = vl / ne;
-    u = first + (vl - ig * ne);
-    return true;
-}
-
 // Fills the context.  row_q(c) returns the e4m3 row of unit column c, row_s(c) its scale row; columns >= nrows
 // alias column 0 (their results are never stored).
 template <typename RowQ, typename RowS>
@@ -533,8 +565,8 @@ __global__ __launch_bounds__(256, 2) void gate_up_prefill_kernel(MfmaArgs a, int
                                                               uint8_t* __restrict__ act_q,
                                                               uint8_t* __restrict__ act_s) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    int u, ig;
-    if (!pf_block_work(a, groups, u, ig)) return;
+    int u, ig, ne;
+    if (!unit_block_work(a, groups, u, ig, ne)) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
@@ -602,8 +634,8 @@ template <typename YT>
 __global__ __launch_bounds__(256, 2) void down_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
                                                            const uint8_t* __restrict__ act_s, YT* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    int u, ig;
-    if (!pf_block_work(a, groups, u, ig)) return;
+    int u, ig, ne;
+    if (!unit_block_work(a, groups, u, ig, ne)) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
@@ -688,8 +720,9 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     static size_t raised = 0;
     int rc = set_lds_limit(gate_up_mfma_kernel<GU_WAVES>, lds, &raised);
     if (rc) return rc;
-    dim3 grid((imax / 32 + GU_WAVES - 1) / GU_WAVES, units.max_units);
-    gate_up_mfma_kernel<GU_WAVES><<<grid, GU_WAVES * 64, lds, st>>>(a, xq, xs, gather_src, act_q, act_s);
+    const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
+    const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+    gate_up_mfma_kernel<GU_WAVES><<<blocks, GU_WAVES * 64, lds, st>>>(a, groups, xq, xs, gather_src, act_q, act_s);
     return check_launch("gate_up_mfma");
 }
 
@@ -711,9 +744,10 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ui
     int rc = set_lds_limit(down_mfma_kernel<DN_WAVES, DN_IPW>, lds, &raised);
     if (rc) return rc;
     const int items = s.hidden / 64;
-    dim3 grid((items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW), units.max_units);
+    const int groups = (items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW);
+    const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
     if (y_dtype != FERRITE_DT_F32) return FERRITE_ERR_INVALID_ARG;
-    down_mfma_kernel<DN_WAVES, DN_IPW><<<grid, DN_WAVES * 64, lds, st>>>(a, act_q, act_s, static_cast<float*>(y));
+    down_mfma_kernel<DN_WAVES, DN_IPW><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
     return check_launch("down_mfma");
 }
 
