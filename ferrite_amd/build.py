@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 SO_PATH = os.path.join(HERE, "libferrite_hip.so")
 SOURCES = ["layer.hip", "route.hip", "formats.hip", "experts_f32.hip", "experts_mfma.hip", "block_ops.hip"]
-HEADERS = ["internal.hpp", "numerics.hpp", "device_utils.hpp"]
+HEADERS = ["internal.hpp", "numerics.hpp", "device_utils.hpp", "prefill_mainloop_asm.inc", "gen_prefill_asm.py"]
 
 
 def source_hash() -> str:

@@ -118,6 +118,33 @@ def test_unit_rows_128_equals_16(hip, oracle, monkeypatch, seed, n, hidden, inte
     assert max_abs_rel(out_bf16, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
 
 
+@pytest.mark.parametrize("seed,n,hidden,inter,shared", [(9, 300, 512, 512, 0), (10, 600, 2048, 512, 512),
+                                                        (11, 1100, 1536, 1024, 512)])
+def test_prefill_assembly_loop_equals_16_row_kernels(hip, oracle, monkeypatch, seed, n, hidden, inter, shared):
+    """FERRITE_HIP_PREFILL=asm selects the 128-row kernels whose main loop is one assembly block (weights streamed
+    through registers, activations through a six-stage LDS ring, counted waits).  Same k order as the 16-row
+    kernels: identical bits with f32 expert outputs, for 1, 4 and 3 groups of four k steps in gate/up (the loop's
+    register and stage rotation repeats every 12 steps) and 1 or 2 in down, ragged units, item groups that are not
+    full; bf16 expert outputs within the MFMA bar of the oracle."""
+    cfg = synth.MoeConfig(n, hidden, 8, 3, inter, shared, 4, 2)
+    inp = synth.make_inputs(cfg, seed=seed)
+    layer = hip.load_moe_layer(inp)
+    monkeypatch.setenv("FERRITE_HIP_Y_F32", "1")
+    monkeypatch.setenv("FERRITE_HIP_UNIT_ROWS", "16")
+    layer._ws.clear()
+    ref16, _ = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    monkeypatch.setenv("FERRITE_HIP_UNIT_ROWS", "128")
+    monkeypatch.setenv("FERRITE_HIP_PREFILL", "asm")
+    layer._ws.clear()
+    got, _ = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    assert np.array_equal(got, ref16)
+    monkeypatch.delenv("FERRITE_HIP_Y_F32")
+    layer._ws.clear()
+    got_bf16, _ = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    layer._ws.clear()
+    assert max_abs_rel(got_bf16, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
+
+
 def test_layer_c1_decode(hip, oracle):
     """The decode benchmark shape: 32 tokens, H 4096, 128 experts, top-8 of 8 groups, I 1536, bf16 activations."""
     inp = synth.make_inputs(synth.CONFIGS["c1"], seed=0)

@@ -27,6 +27,14 @@ def test_library_exports_every_declared_symbol():
     assert lib.ferrite_kernel_build_id().decode().startswith("ferrite-hip-")
 
 
+def test_generated_assembly_loop_is_current(tmp_path):
+    """csrc/prefill_mainloop_asm.inc is what csrc/gen_prefill_asm.py writes."""
+    csrc = os.path.join(ROOT, "ferrite_amd", "csrc")
+    out = str(tmp_path / "loop.inc")
+    subprocess.run([os.sys.executable, os.path.join(csrc, "gen_prefill_asm.py"), out], check=True, capture_output=True)
+    assert open(out).read() == open(os.path.join(csrc, "prefill_mainloop_asm.inc")).read()
+
+
 def test_backend_refuses_to_run_without_gpu_or_library(tmp_path):
     import torch
     from ferrite_amd import backend
