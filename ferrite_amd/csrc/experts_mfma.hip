@@ -408,9 +408,12 @@ __global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, int g
 // barrier, operand reads) hides behind the other's MFMAs.
 // Accumulation order over k is the same as in the 16-row kernels, so both give the same bits.
 constexpr int PF_ROWS = 128;
-constexpr int PF_ITEMS = 4;
-constexpr int PF_LDS_STAGE = 2 * 1024;                 // u4v per stage: 1024 weight slots + 1024 activation slots
-constexpr size_t PF_LDS_BYTES = 2 * PF_LDS_STAGE * 16;  // 64 KiB
+constexpr int PF_ITEMS = 4;                            // 8 (one block of 8 waves per CU) is correct too and measured slower
+constexpr int PF_WAVES = PF_ITEMS;                     // one wave per item for the fills; 2 items x 64 rows each for the MFMAs
+constexpr int PF_A_SLOTS = PF_ITEMS * 256;             // u4v of weights per stage
+constexpr int PF_LDS_STAGE = PF_A_SLOTS + 1024;        // + 1024 activation slots
+constexpr size_t PF_LDS_BYTES = 2 * PF_LDS_STAGE * 16;  // 64 KiB (4 items) / 96 KiB (8 items)
+constexpr int PR_ITEMS = 4;
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void glb_void;
@@ -433,11 +436,12 @@ __device__ __forceinline__ void pf_fill(const PfCtx& c, u4v* stage, int kt) {
     const u4v* a = c.a_src + (size_t)kt * 256;
 #pragma unroll
     for (int t = 0; t < 4; ++t) dma16(a + t * 64, stage + (c.wave * 4 + t) * 64);
+    constexpr int NB = 16 / PF_WAVES;   // half tiles of activations per wave
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-            dma16(c.b_src[i] + (size_t)kt * 128 + h * 64, stage + 1024 + ((c.wave * 2 + i) * 2 + h) * 64);
+    for (int j = 0; j < NB; ++j) {
+        const int i = j >> 1, h = j & 1;   // NB 4: tiles 2w, 2w+1 x halves; NB 2: tile w x halves
+        dma16(c.b_src[i] + (size_t)kt * 128 + h * 64, stage + PF_A_SLOTS + (c.wave * NB + j) * 64);
+    }
 }
 
 // All loads into LDS issued by this wave have landed (vmcnt 0; expcnt and lgkmcnt left alone).
@@ -454,7 +458,7 @@ __device__ __forceinline__ void pf_step(const PfCtx& c, u4v* lds, int kt, const 
     u4v av[2][4];
 #pragma unroll
     for (int tt = 0; tt < 4; ++tt) {
-        const u4v* bt = cur + 1024 + (c.wt * 4 + tt) * 128 + c.bslot;
+        const u4v* bt = cur + PF_A_SLOTS + (c.wt * 4 + tt) * 128 + c.bslot;
         const u4v b0 = bt[0];
         const u4v b1 = bt[64];
         bv[tt] = (v8i){(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
@@ -534,7 +538,7 @@ __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const
     c.KT = KT;
     c.lane = threadIdx.x & 63;
     c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    c.wi = c.wave & 1; c.wt = c.wave >> 1;
+    c.wi = c.wave % (PF_ITEMS / 2); c.wt = c.wave / (PF_ITEMS / 2);
     const int cc = c.lane & 15, g = c.lane >> 4;
     c.a_src = reinterpret_cast<const u4v*>(cbase) + (size_t)min(item0 + c.wave, items - 1) * KT * 256 + c.lane;
     // Activation stage layout: the four lanes of a quad fetch 64 consecutive bytes of one row (what the texture
@@ -543,7 +547,7 @@ __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const
     // chunk) touch eight different 16-byte bank groups (counters: no LDS bank conflicts; XOR with r/4 had them).
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-        const int col = (c.wave * 2 + i) * 16 + (c.lane >> 2);
+        const int col = (PF_WAVES == 4 ? c.wave * 2 + i : c.wave) * 16 + (c.lane >> 2);
         c.b_src[i] = row_q(col < nrows ? col : 0) + ((c.lane & 3) ^ ((c.lane >> 3) & 3)) * 16;
     }
     c.bslot = 4 * cc + (g ^ ((cc >> 1) & 3));
@@ -559,7 +563,7 @@ __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const
     }
 }
 
-__global__ __launch_bounds__(256, 2) void gate_up_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
+__global__ __launch_bounds__(PF_WAVES * 64, PF_WAVES == 4 ? 2 : 1) void gate_up_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
                                                               const uint8_t* __restrict__ xs,
                                                               const int32_t* __restrict__ gather_src,
                                                               uint8_t* __restrict__ act_q,
@@ -631,7 +635,7 @@ __device__ __forceinline__ uint32_t bf16_rne(float f) {
 }
 
 template <typename YT>
-__global__ __launch_bounds__(256, 2) void down_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
+__global__ __launch_bounds__(PF_WAVES * 64, PF_WAVES == 4 ? 2 : 1) void down_prefill_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
                                                            const uint8_t* __restrict__ act_s, YT* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig, ne;
@@ -795,7 +799,7 @@ __global__ __launch_bounds__(256, 1) void gate_up_pr_kernel(MfmaArgs a, int grou
     if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
     const int inter = shared ? a.shared_inter : a.inter;
-    const int items = inter / 32, item0 = ig * PF_ITEMS;
+    const int items = inter / 32, item0 = ig * PR_ITEMS;
     if (item0 >= items) return;
     const int H = a.hidden, nk = a.n * a.topk, topk = a.topk, n = a.n;
     const int spitch = scale_pitch(H);
@@ -850,7 +854,7 @@ __global__ __launch_bounds__(256, 1) void down_pr_kernel(MfmaArgs a, int groups,
     if (!unit_ok(a, e, row0, nrows)) return;
     const bool shared = e == a.n_experts;
     const int inter = shared ? a.shared_inter : a.inter;
-    const int H = a.hidden, items = H / 64, item0 = ig * PF_ITEMS;
+    const int H = a.hidden, items = H / 64, item0 = ig * PR_ITEMS;
     if (item0 >= items) return;
     const int apitch = scale_pitch(a.act_ld), act_ld = a.act_ld;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -910,9 +914,11 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     MfmaArgs a = make_args(s, packed, n, units, false);
     const int imax = a.act_ld;
     if (units.unit_rows_cap == PF_ROWS) {
-        const int groups = (imax / 32 + PF_ITEMS - 1) / PF_ITEMS;
+        const bool asm_loop = prefill_asm_loop(s.hidden);
+        const int ipb = asm_loop ? PR_ITEMS : PF_ITEMS;   // items per block
+        const int groups = (imax / 32 + ipb - 1) / ipb;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-        if (prefill_asm_loop(s.hidden)) {
+        if (asm_loop) {
             static size_t raised_pr = 0;
             const size_t lds = pr_lds_bytes(s.hidden);
             int rc = set_lds_limit(gate_up_pr_kernel, lds, &raised_pr);
@@ -923,7 +929,7 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
         static size_t raised_pf = 0;
         int rc = set_lds_limit(gate_up_prefill_kernel, PF_LDS_BYTES, &raised_pf);
         if (rc) return rc;
-        gate_up_prefill_kernel<<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, xq, xs, gather_src, act_q, act_s);
+        gate_up_prefill_kernel<<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, xq, xs, gather_src, act_q, act_s);
         return check_launch("gate_up_prefill");
     }
     if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
@@ -941,10 +947,12 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ui
                      int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
     MfmaArgs a = make_args(s, packed, n, units, true);
     if (units.unit_rows_cap == PF_ROWS) {
-        const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
-        const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
         // every expert of the launch must qualify: routed and shared intermediate sizes
-        if (prefill_asm_loop(s.inter) && (s.shared_inter == 0 || prefill_asm_loop(s.shared_inter))) {
+        const bool asm_loop = prefill_asm_loop(s.inter) && (s.shared_inter == 0 || prefill_asm_loop(s.shared_inter));
+        const int ipb = asm_loop ? PR_ITEMS : PF_ITEMS;
+        const int groups = (s.hidden / 64 + ipb - 1) / ipb;
+        const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+        if (asm_loop) {
             const size_t lds = pr_lds_bytes(a.act_ld);
             int rc;
             if (y_dtype == FERRITE_DT_BF16) {
@@ -958,10 +966,16 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ui
             }
             return check_launch("down_pr");
         }
-        if (y_dtype == FERRITE_DT_BF16)
-            down_prefill_kernel<uint16_t><<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<uint16_t*>(y));
-        else
-            down_prefill_kernel<float><<<blocks, 256, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
+        int rc;
+        if (y_dtype == FERRITE_DT_BF16) {
+            static size_t raised = 0;
+            if ((rc = set_lds_limit(down_prefill_kernel<uint16_t>, PF_LDS_BYTES, &raised))) return rc;
+            down_prefill_kernel<uint16_t><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<uint16_t*>(y));
+        } else {
+            static size_t raised = 0;
+            if ((rc = set_lds_limit(down_prefill_kernel<float>, PF_LDS_BYTES, &raised))) return rc;
+            down_prefill_kernel<float><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
+        }
         return check_launch("down_prefill");
     }
     if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
