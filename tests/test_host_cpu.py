@@ -27,6 +27,16 @@ def test_library_exports_every_declared_symbol():
     assert lib.ferrite_kernel_build_id().decode().startswith("ferrite-hip-")
 
 
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits before touching a device."""
+    for extra_env in ({}, {"WORLD_SIZE": "2"}):
+        env = dict(os.environ, **extra_env)
+        args = [os.sys.executable, os.path.join(ROOT, "bench.py")] + ([] if extra_env else ["--gpus", "2"])
+        res = subprocess.run(args, capture_output=True, text=True, env=env, timeout=60)
+        assert res.returncode == 2
+        assert "one GPU" in res.stderr and res.stdout == ""
+
+
 def test_generated_assembly_loop_is_current(tmp_path):
     """csrc/prefill_mainloop_asm.inc is what csrc/gen_prefill_asm.py writes."""
     csrc = os.path.join(ROOT, "ferrite_amd", "csrc")
