@@ -123,50 +123,80 @@ __global__ __launch_bounds__(256) void down_f32_kernel(ferrite_moe_shape s, ferr
 
 // out[t] = sum_j (ascending) probs[t,j] * y[perm_map[t*k+j]]  then  + y[n*k + t]   (exec/lib.rs:1154-1164:
 // a rounded product and a rounded add per slot, the shared expert last)
-// four consecutive y values of a row: f32, or bf16 widened (exact)
+// One 16-byte piece of a y row: four f32, or eight bf16 widened (exact).
 template <typename YT>
-__device__ __forceinline__ float4 load_y4(const YT* p) {
-    if constexpr (sizeof(YT) == 4) {
-        return *reinterpret_cast<const float4*>(p);
-    } else {
-        const uint2 q = *reinterpret_cast<const uint2*>(p);
-        return make_float4(u2f(q.x << 16), u2f(q.x & 0xffff0000u), u2f(q.y << 16), u2f(q.y & 0xffff0000u));
+struct YPiece {
+    static constexpr int N = 16 / sizeof(YT);
+    uint4 raw;
+    __device__ __forceinline__ float at(int i) const {
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        if constexpr (sizeof(YT) == 4) return u2f(w[i]);
+        else return u2f((i & 1) ? (w[i >> 1] & 0xffff0000u) : (w[i >> 1] << 16));
     }
+};
+
+// f32 -> bf16, round to nearest even (NaN stays NaN)
+__device__ __forceinline__ uint32_t combine_bf16(float f) {
+    const uint32_t u = f2u(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
 }
 
+// A thread owns 16 bytes of every y row of its token (4 or 8 columns).  The slots are walked in batches of eight:
+// first the eight table entries, then the eight row pieces - all loads of a batch are in flight together - then the
+// products and sums in slot order.
 template <typename OT, typename YT>
 __global__ __launch_bounds__(256) void combine_kernel(const YT* __restrict__ y, const float* __restrict__ probs,
                                                       const int32_t* __restrict__ perm_map, int n, int topk,
                                                       int H, int has_shared, OT* __restrict__ out) {
+    constexpr int N = YPiece<YT>::N;
     const int t = blockIdx.y;
-    const int h = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    const int h = (blockIdx.x * blockDim.x + threadIdx.x) * N;
     if (h >= H) return;
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int j = 0; j < topk; ++j) {
-        int g = perm_map[(size_t)t * topk + j];
-        if (g < 0 || g >= n * topk) continue;   // tables of an uninitialised workspace must not cause a fault
-        float p = probs[(size_t)t * topk + j];
-        float4 v = load_y4(y + (size_t)g * H + h);
-        o.x = fadd(o.x, fmul(p, v.x)); o.y = fadd(o.y, fmul(p, v.y));
-        o.z = fadd(o.z, fmul(p, v.z)); o.w = fadd(o.w, fmul(p, v.w));
+    float o[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) o[i] = 0.0f;
+    const int nk = n * topk;
+    for (int j0 = 0; j0 < topk; j0 += 8) {
+        int g[8];
+        float p[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bool in = j0 + j < topk;
+            g[j] = in ? perm_map[(size_t)t * topk + j0 + j] : -1;
+            p[j] = in ? probs[(size_t)t * topk + j0 + j] : 0.0f;
+        }
+        YPiece<YT> v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            // tables of an uninitialised workspace must not cause a fault: such slots are skipped
+            const bool ok = g[j] >= 0 && g[j] < nk;
+            v[j].raw = ok ? *reinterpret_cast<const uint4*>(y + (size_t)g[j] * H + h) : make_uint4(0u, 0u, 0u, 0u);
+            g[j] = ok ? 1 : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (g[j]) {
+#pragma unroll
+                for (int i = 0; i < N; ++i) o[i] = fadd(o[i], fmul(p[j], v[j].at(i)));
+            }
+        }
     }
     if (has_shared) {
-        float4 v = load_y4(y + ((size_t)n * topk + t) * H + h);
-        o.x = fadd(o.x, v.x); o.y = fadd(o.y, v.y); o.z = fadd(o.z, v.z); o.w = fadd(o.w, v.w);
+        YPiece<YT> v;
+        v.raw = *reinterpret_cast<const uint4*>(y + ((size_t)nk + t) * H + h);
+#pragma unroll
+        for (int i = 0; i < N; ++i) o[i] = fadd(o[i], v.at(i));
     }
+    OT* dst = out + (size_t)t * H + h;
     if constexpr (sizeof(OT) == 4) {
-        *reinterpret_cast<float4*>(out + (size_t)t * H + h) = o;
+#pragma unroll
+        for (int i = 0; i < N; i += 4) *reinterpret_cast<float4*>(dst + i) = make_float4(o[i], o[i + 1], o[i + 2], o[i + 3]);
     } else {
-        // f32 -> bf16 round to nearest even
-        auto cv = [](float f) -> uint32_t {
-            uint32_t u = f2u(f);
-            if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-            return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-        };
-        uint2 pk;
-        pk.x = cv(o.x) | (cv(o.y) << 16);
-        pk.y = cv(o.z) | (cv(o.w) << 16);
-        *reinterpret_cast<uint2*>(out + (size_t)t * H + h) = pk;
+#pragma unroll
+        for (int i = 0; i < N; i += 4)
+            *reinterpret_cast<uint2*>(dst + i) = make_uint2(combine_bf16(o[i]) | (combine_bf16(o[i + 1]) << 16),
+                                                            combine_bf16(o[i + 2]) | (combine_bf16(o[i + 3]) << 16));
     }
 }
 
@@ -190,8 +220,10 @@ int launch_down_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, co
 
 int launch_combine(const void* y, int y_dtype, const float* probs, const int32_t* perm_map, int n, int topk,
                    int hidden, int has_shared, void* out, int out_dtype, hipStream_t st) {
-    dim3 grid((hidden / 4 + 255) / 256, n);
     const bool of32 = out_dtype == FERRITE_DT_F32, yf32 = y_dtype == FERRITE_DT_F32;
+    const int per_thread = yf32 ? 4 : 8;   // columns per thread: 16 bytes of a y row
+    if (hidden % per_thread) return FERRITE_ERR_INVALID_ARG;
+    dim3 grid((hidden / per_thread + 255) / 256, n);
     if ((!of32 && out_dtype != FERRITE_DT_BF16) || (!yf32 && y_dtype != FERRITE_DT_BF16)) return FERRITE_ERR_INVALID_ARG;
     if (of32 && yf32)
         combine_kernel<float, float><<<grid, 256, 0, st>>>((const float*)y, probs, perm_map, n, topk, hidden, has_shared, (float*)out);
