@@ -21,7 +21,7 @@ from .backend import DEFAULT_SO, FerriteError, HipBackend, InvalidArg, MoeConfig
 
 HOST_SO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "host", "libferrite_host.so")
 NAMING_DSV41, NAMING_GLM = 0, 1
-HOST_EXPORTS = ["ferrite_ckpt_open", "ferrite_ckpt_close", "ferrite_ckpt_num_tensors", "ferrite_ckpt_data_start",
+HOST_EXPORTS = ["ferrite_ckpt_open", "ferrite_ckpt_add_shard", "ferrite_ckpt_close", "ferrite_ckpt_num_tensors", "ferrite_ckpt_data_start",
                 "ferrite_ckpt_tensor", "ferrite_ckpt_validate_moe", "ferrite_ckpt_load_moe_layer"]
 
 
@@ -33,6 +33,7 @@ def load_host_library(so_path: Optional[str] = None) -> C.CDLL:
     vp, i32, sz, cp = C.c_void_p, C.c_int, C.c_size_t, C.c_char_p
     lib.ferrite_ckpt_open.restype = vp
     lib.ferrite_ckpt_open.argtypes = [cp, cp, sz]
+    lib.ferrite_ckpt_add_shard.argtypes = [vp, cp, cp, sz]
     lib.ferrite_ckpt_close.restype = None
     lib.ferrite_ckpt_close.argtypes = [vp]
     lib.ferrite_ckpt_num_tensors.restype = C.c_int64
@@ -65,15 +66,26 @@ class LoadStats:
 
 
 class Checkpoint:
-    """One opened safetensors shard: header index + read-only mapping."""
+    """An opened checkpoint: one safetensors file, or the shards of a split one (header indexes + read-only
+    mappings; a tensor is taken from the first shard that names it)."""
 
-    def __init__(self, path: str, host_so: Optional[str] = None):
+    def __init__(self, path, host_so: Optional[str] = None):
+        paths = [path] if isinstance(path, (str, bytes, os.PathLike)) else list(path)
+        if not paths:
+            raise InvalidArg("no checkpoint file given")
         self.lib = load_host_library(host_so)
+        self._h = None
         err = C.create_string_buffer(512)
-        self._h = self.lib.ferrite_ckpt_open(os.fsencode(path), err, len(err))
+        self._h = self.lib.ferrite_ckpt_open(os.fsencode(paths[0]), err, len(err))
         if not self._h:
             raise InvalidArg(err.value.decode(errors="replace"))
-        self.path = path
+        for p in paths[1:]:
+            if self.lib.ferrite_ckpt_add_shard(self._h, os.fsencode(p), err, len(err)) != 0:
+                msg = err.value.decode(errors="replace")
+                self.close()
+                raise InvalidArg(msg)
+        self.path = paths[0]
+        self.paths = paths
 
     def close(self):
         if self._h:
@@ -182,9 +194,10 @@ def moe_tensor_names(naming: int, prefix: str, expert: int, n_experts: int) -> D
     return {"gate": f"{p}.gate_proj", "up": f"{p}.up_proj", "down": f"{p}.down_proj"}
 
 
-def write_moe_checkpoint(path: str, inp, prefix: str, naming: int = NAMING_DSV41,
-                         values: Optional[Dict[str, np.ndarray]] = None, value_tag: str = "BF16") -> None:
-    """One layer's MoE as a checkpoint shard.  NAMING_DSV41 writes `inp`'s MXFP4 tensors as they are (I8 codes,
+def moe_checkpoint_tensors(inp, prefix: str, naming: int = NAMING_DSV41,
+                           values: Optional[Dict[str, np.ndarray]] = None,
+                           value_tag: str = "BF16") -> List[Tuple[str, str, np.ndarray]]:
+    """One layer's MoE as (name, dtype tag, array) triples in checkpoint order.  NAMING_DSV41 writes `inp`'s MXFP4 tensors as they are (I8 codes,
     F8_E8M0 scales); NAMING_GLM writes unquantised matrices taken from `values` (name stem -> [out, in] array of
     the numpy type that `value_tag` stands for)."""
     cfg = inp.cfg
@@ -205,4 +218,10 @@ def write_moe_checkpoint(path: str, inp, prefix: str, naming: int = NAMING_DSV41
         else:
             for key in ("gate", "down", "up"):
                 out.append((nm[key] + ".weight", value_tag, values[nm[key]]))
-    write_safetensors(path, out, metadata={"format": "pt"})
+    return out
+
+
+def write_moe_checkpoint(path: str, inp, prefix: str, naming: int = NAMING_DSV41,
+                         values: Optional[Dict[str, np.ndarray]] = None, value_tag: str = "BF16") -> None:
+    """One layer's MoE as a single checkpoint file (see moe_checkpoint_tensors)."""
+    write_safetensors(path, moe_checkpoint_tensors(inp, prefix, naming, values, value_tag), metadata={"format": "pt"})

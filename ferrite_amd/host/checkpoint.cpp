@@ -431,10 +431,20 @@ struct MatSrc {
 
 struct ExpertSrc { MatSrc gate, up, down; };
 
-const uint8_t* tensor_bytes(const MappedFile& f, const SafetensorsIndex& idx, const std::string& name,
+// The shard of a set that holds `name` (the first one that does), or null.
+const CheckpointShard* shard_of(const std::vector<CheckpointShard>& shards, const std::string& name) {
+    for (const CheckpointShard& sh : shards)
+        if (sh.index->find(name)) return &sh;
+    return nullptr;
+}
+
+const uint8_t* tensor_bytes(const std::vector<CheckpointShard>& shards, const std::string& name,
                             const std::vector<std::string>& dtypes, const std::vector<size_t>& shape, size_t* esize) {
+    const CheckpointShard* sh = shard_of(shards, name);
+    if (!sh) config_error("missing tensor " + name);
+    const MappedFile& f = *sh->file;
+    const SafetensorsIndex& idx = *sh->index;
     const TensorView* v = idx.find(name);
-    if (!v) config_error("missing tensor " + name);
     bool dt_ok = false;
     for (const auto& d : dtypes) dt_ok = dt_ok || d == v->dtype;
     if (!dt_ok) config_error(name + ": dtype " + v->dtype + " is not one this path loads");
@@ -461,6 +471,16 @@ void copy_plane(uint8_t* dst, const uint8_t* src, size_t rows, size_t cols, size
 LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const SafetensorsIndex& index, MoeNaming naming,
                                           const std::string& prefix, const ferrite_moe_shape& s, uint8_t* packed_dev,
                                           float* router_bias_dev, const LoadOptions& opt) const {
+    return load_layer(std::vector<CheckpointShard>{CheckpointShard{&file, &index}}, naming, prefix, s, packed_dev,
+                      router_bias_dev, opt);
+}
+
+LoadStats MoeCheckpointLoader::load_layer(const std::vector<CheckpointShard>& shards, MoeNaming naming,
+                                          const std::string& prefix, const ferrite_moe_shape& s, uint8_t* packed_dev,
+                                          float* router_bias_dev, const LoadOptions& opt) const {
+    if (shards.empty()) config_error("no checkpoint shard given");
+    for (const CheckpointShard& sh : shards)
+        if (!sh.file || !sh.index) config_error("null checkpoint shard");
     const auto t0 = std::chrono::steady_clock::now();
     if (!packed_dev) config_error("packed_dev is null");
     const size_t pbytes = api_->ferrite_moe_packed_bytes(&s);
@@ -474,12 +494,12 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
     LoadStats stats;
     stats.packed_bytes = pbytes;
     size_t router_es = 0;
-    const uint8_t* router_src = tensor_bytes(file, index, prefix + ".gate.weight", val_dt, {E, H}, &router_es);
+    const uint8_t* router_src = tensor_bytes(shards, prefix + ".gate.weight", val_dt, {E, H}, &router_es);
     stats.source_bytes += E * H * router_es;
     const uint8_t* bias_src = nullptr;
     size_t bias_es = 0;
-    if (index.find(bias_name(naming, prefix))) {
-        bias_src = tensor_bytes(file, index, bias_name(naming, prefix), val_dt, {E}, &bias_es);
+    if (shard_of(shards, bias_name(naming, prefix))) {
+        bias_src = tensor_bytes(shards, bias_name(naming, prefix), val_dt, {E}, &bias_es);
         stats.source_bytes += E * bias_es;
         if (!router_bias_dev) config_error("the checkpoint has a routing bias but router_bias_dev is null");
     }
@@ -490,7 +510,8 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
         const size_t I = e == s.n_experts ? s.shared_inter : s.inter;
         const std::string p = expert_prefix(naming, prefix, e, s.n_experts);
         if (quantised && e == s.n_experts) {
-            const TensorView* v = index.find(p + "." + mn.gate + ".weight");
+            const CheckpointShard* sh = shard_of(shards, p + "." + mn.gate + ".weight");
+            const TensorView* v = sh ? sh->index->find(p + "." + mn.gate + ".weight") : nullptr;
             if (v && v->dtype == "F8_E4M3")
                 config_error(p + ": the shared expert is stored as F8_E4M3, which is not an MXFP4 tensor; load the layer "
                              "with shared_inter = 0 and run the shared expert on its own path");
@@ -499,13 +520,13 @@ LoadStats MoeCheckpointLoader::load_layer(const MappedFile& file, const Safetens
             MatSrc m;
             m.rows = o; m.cols = k;
             if (quantised) {
-                m.w = tensor_bytes(file, index, p + "." + nm + ".weight", code_dt, {o, k / 2}, nullptr);
-                m.s = tensor_bytes(file, index, p + "." + nm + ".scale", scale_dt, {o, k / 32}, nullptr);
+                m.w = tensor_bytes(shards, p + "." + nm + ".weight", code_dt, {o, k / 2}, nullptr);
+                m.s = tensor_bytes(shards, p + "." + nm + ".scale", scale_dt, {o, k / 32}, nullptr);
                 m.w_bytes = o * k / 2;
                 m.esize = 1;
                 stats.source_bytes += m.w_bytes + o * k / 32;
             } else {
-                m.w = tensor_bytes(file, index, p + "." + nm + ".weight", val_dt, {o, k}, &m.esize);
+                m.w = tensor_bytes(shards, p + "." + nm + ".weight", val_dt, {o, k}, &m.esize);
                 m.w_bytes = o * k * m.esize;
                 stats.source_bytes += m.w_bytes;
             }

@@ -81,6 +81,12 @@ std::vector<TensorSpec> moe_layer_specs(MoeNaming naming, const std::string& pre
 // the checkpoint layout on the device: rows padded to the next multiple of 16 bytes (weights.rs:599).
 inline size_t sf_plane_pitch(size_t cols) { return (cols + 15) & ~size_t(15); }
 
+// One shard of a checkpoint that is split over several files (both pointers borrowed).
+struct CheckpointShard {
+    const MappedFile* file;
+    const SafetensorsIndex* index;
+};
+
 struct LoadStats {
     uint64_t source_bytes = 0;   // bytes of the layer's tensors read from the file
     uint64_t packed_bytes = 0;   // size of the packed buffer
@@ -107,6 +113,11 @@ class MoeCheckpointLoader {
     LoadStats load_layer(const MappedFile& file, const SafetensorsIndex& index, MoeNaming naming,
                          const std::string& prefix, const ferrite_moe_shape& shape, uint8_t* packed_dev,
                          float* router_bias_dev, const LoadOptions& opt = LoadOptions()) const;
+    // The same over a checkpoint split into shards: every tensor is taken from the first shard that names it (a
+    // layer's experts usually straddle two or three files of a released checkpoint).
+    LoadStats load_layer(const std::vector<CheckpointShard>& shards, MoeNaming naming, const std::string& prefix,
+                         const ferrite_moe_shape& shape, uint8_t* packed_dev, float* router_bias_dev,
+                         const LoadOptions& opt = LoadOptions()) const;
 
   private:
     struct Api;

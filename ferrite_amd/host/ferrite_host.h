@@ -22,6 +22,9 @@ extern "C" {
 typedef struct ferrite_ckpt ferrite_ckpt; /* an opened shard: header index + read-only mapping */
 
 ferrite_ckpt* ferrite_ckpt_open(const char* path, char* err, size_t errlen);
+/* A checkpoint split over several files: further shards of the same checkpoint.  A tensor is taken from the first
+ * shard that names it; ferrite_ckpt_data_start() is that of the first shard. */
+int ferrite_ckpt_add_shard(ferrite_ckpt* ck, const char* path, char* err, size_t errlen);
 void ferrite_ckpt_close(ferrite_ckpt* ck);
 int64_t ferrite_ckpt_num_tensors(const ferrite_ckpt* ck);
 uint64_t ferrite_ckpt_data_start(const ferrite_ckpt* ck);

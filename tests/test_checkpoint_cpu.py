@@ -187,3 +187,25 @@ def test_moe_names_glm(tmp_path):
             assert c.tensor(name) is not None, name
         assert c.tensor("model.layers.3.mlp.experts.1.up_proj.weight").shape == (cfg.inter, cfg.hidden)
         assert c.validate_moe(cfg, "model.layers.3.mlp", ck.NAMING_GLM) == []
+
+
+def test_split_checkpoint_takes_each_tensor_from_the_shard_that_names_it(tmp_path):
+    cfg = _tiny_cfg()
+    inp = synth.make_inputs(cfg, seed=0)
+    tensors = ck.moe_checkpoint_tensors(inp, "layers.6.ffn", ck.NAMING_DSV41)
+    paths = [str(tmp_path / f"model-{i:05d}-of-00003.safetensors") for i in range(3)]
+    for i, p in enumerate(paths):                       # tensors dealt round-robin over three files
+        ck.write_safetensors(p, tensors[i::3], metadata={"format": "pt"})
+    with ck.Checkpoint(paths) as c:
+        assert len(c) == len(tensors)
+        assert c.validate_moe(cfg, "layers.6.ffn", ck.NAMING_DSV41) == []
+        for name, tag, arr in tensors:
+            v = c.tensor(name)
+            assert (v.dtype, v.shape) == (tag, arr.shape), name
+    with ck.Checkpoint(paths[:2]) as c:                  # a shard short: its tensors are reported by name
+        missing = c.validate_moe(cfg, "layers.6.ffn", ck.NAMING_DSV41)
+        assert sorted(missing) == sorted(n for n, _, _ in tensors[2::3])
+    with pytest.raises(InvalidArg, match=r"^open .*absent\.safetensors: "):
+        ck.Checkpoint([paths[0], str(tmp_path / "absent.safetensors")])
+    with pytest.raises(InvalidArg):
+        ck.Checkpoint([])

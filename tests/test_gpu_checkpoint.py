@@ -73,6 +73,25 @@ def test_dsv41_shard_loads_into_the_same_packed_bytes(hip, oracle, tmp_path, wor
     assert torch.equal(out_a, out_b)
 
 
+def test_split_checkpoint_loads_like_a_single_file(hip, tmp_path):
+    """The layer's tensors dealt over three shard files (as released checkpoints split a layer's experts) load
+    into the same packed bytes."""
+    cfg = _cfg()
+    inp = synth.make_inputs(cfg, seed=15)
+    ref_layer = hip.load_moe_layer(inp)
+    tensors = ck.moe_checkpoint_tensors(inp, "layers.6.ffn", ck.NAMING_DSV41)
+    paths = [str(tmp_path / f"model-{i:05d}-of-00003.safetensors") for i in range(3)]
+    for i, p in enumerate(paths):
+        ck.write_safetensors(p, tensors[i::3])
+    with ck.Checkpoint(paths) as c:
+        layer, stats = c.load_moe_layer(hip, cfg, "layers.6.ffn", ck.NAMING_DSV41, workers=5)
+    assert torch.equal(layer.packed, ref_layer.packed)
+    assert stats.source_bytes == sum(a.nbytes for _, _, a in tensors)
+    with ck.Checkpoint(paths[1:]) as c:
+        with pytest.raises(InvalidArg, match="missing tensor layers.6.ffn.gate.weight"):
+            c.load_moe_layer(hip, cfg, "layers.6.ffn", ck.NAMING_DSV41)
+
+
 def test_pack_expert_with_padded_scale_rows(hip, oracle):
     """The source pitch argument: scale planes staged with rows padded to 16 bytes (weights.rs:599) and filled with
     junk between the rows give the same packed bytes as dense planes."""
