@@ -246,13 +246,15 @@ def main():
     # per-stage durations: eager launches with HIP events recorded on the launch stream between the stages
     ev = HipEvents()
     k_prof = min(args.steps, 50)
-    sets = [ev.create(8) for _ in range(k_prof)]
+    sets = [ev.create(10) for _ in range(k_prof)]
     for s in sets:
         hip.moe_layer_dev_mxfp4(layer, x, out, MODE_MFMA_FP8, ws, stage_events=s)
     hip.sync()
     names = ["router_gemm", "route", "permute", "act_quant", "gate_up_mfma", "down_mfma", "combine"]
     stage_us = {nm: float(np.mean([ev.elapsed_ms(s[i], s[i + 1]) for s in sets]) * 1e3) for i, nm in enumerate(names)}
     eager_us = float(np.mean([ev.elapsed_ms(s[0], s[7]) for s in sets]) * 1e3)
+    # the gate/up kernel itself: events that bracket its execution on the device (what rocprofv3 reports)
+    gu_kernel_us = float(np.mean([ev.elapsed_ms(s[8], s[9]) for s in sets]) * 1e3)
     for s in sets:
         ev.destroy(s)
 
@@ -264,7 +266,7 @@ def main():
 
     us_layer = ms_per_step * 1e3 / n_layers
     unit_rows = hip.unit_rows(layer, n, MODE_MFMA_FP8)
-    gu_us = stage_us["gate_up_mfma"]
+    gu_us = gu_kernel_us
     if unit_rows == 16:
         # decode-sized batch: every weight byte is streamed once per 16-row unit; the kernel is HBM bound
         gate_up_gbs = ab["gate_up"] / (gu_us * 1e-6) / 1e9

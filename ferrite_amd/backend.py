@@ -61,6 +61,9 @@ class MoeWeights(C.Structure):
     _fields_ = [(k, C.c_void_p) for k in _WEIGHT_FIELDS]
 
 
+STAGE_EVENTS = 10   # FERRITE_MOE_STAGE_EVENTS
+
+
 class MoeExpertSrc(C.Structure):
     _fields_ = [(k, C.c_void_p) for k in ("gate_w", "gate_s", "up_w", "up_s", "down_w", "down_s")] + \
                [("gate_up_scale_pitch", C.c_int64), ("down_scale_pitch", C.c_int64)]
@@ -527,6 +530,8 @@ class HipBackend:
         if stage_events is None:
             self._ck(self.lib.ferrite_moe_layer_mxfp4(*args), "moe_layer_mxfp4")
         else:
+            if len(stage_events) != STAGE_EVENTS:
+                raise InvalidArg(f"stage_events must hold {STAGE_EVENTS} event handles")
             self._ck(self.lib.ferrite_moe_layer_mxfp4_timed(*args, stage_events), "moe_layer_mxfp4")
 
     def block_workspace(self, layer: MoeLayer, n: int, mode: int) -> torch.Tensor:

@@ -12,6 +12,8 @@
 // The packed weight buffer stores, per work item (32 gate rows + the same 32 up rows, or 64 down rows), the
 // code tiles in exactly the order a wave consumes them: [item][k step][tile 0..3][lane][16 B], so a wave
 // reads one contiguous 4 KiB per k step with 128-bit loads; scales are [item][4 k steps][lane][tile][4 B].
+#include <hip/hip_ext.h>
+
 #include "internal.hpp"
 #include "device_utils.hpp"
 #include "numerics.hpp"
@@ -908,9 +910,10 @@ static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int
     return a;
 }
 
+// k_start / k_stop (may be null): events that bracket the kernel itself on the device, not the launch.
 int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
                         int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
-                        hipStream_t st) {
+                        hipStream_t st, hipEvent_t k_start, hipEvent_t k_stop) {
     MfmaArgs a = make_args(s, packed, n, units, false);
     const int imax = a.act_ld;
     if (units.unit_rows_cap == PF_ROWS) {
@@ -923,13 +926,15 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
             const size_t lds = pr_lds_bytes(s.hidden);
             int rc = set_lds_limit(gate_up_pr_kernel, lds, &raised_pr);
             if (rc) return rc;
-            gate_up_pr_kernel<<<blocks, 256, lds, st>>>(a, groups, xq, xs, gather_src, act_q, act_s);
+            hipExtLaunchKernelGGL(gate_up_pr_kernel, dim3(blocks), dim3(256), (uint32_t)lds, st, k_start, k_stop, 0, a, groups,
+                                  xq, xs, gather_src, act_q, act_s);
             return check_launch("gate_up_pr");
         }
         static size_t raised_pf = 0;
         int rc = set_lds_limit(gate_up_prefill_kernel, PF_LDS_BYTES, &raised_pf);
         if (rc) return rc;
-        gate_up_prefill_kernel<<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, xq, xs, gather_src, act_q, act_s);
+        hipExtLaunchKernelGGL(gate_up_prefill_kernel, dim3(blocks), dim3(PF_WAVES * 64), (uint32_t)PF_LDS_BYTES, st, k_start,
+                              k_stop, 0, a, groups, xq, xs, gather_src, act_q, act_s);
         return check_launch("gate_up_prefill");
     }
     if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
@@ -939,7 +944,8 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     if (rc) return rc;
     const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
     const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-    gate_up_mfma_kernel<GU_WAVES><<<blocks, GU_WAVES * 64, lds, st>>>(a, groups, xq, xs, gather_src, act_q, act_s);
+    hipExtLaunchKernelGGL(gate_up_mfma_kernel<GU_WAVES>, dim3(blocks), dim3(GU_WAVES * 64), (uint32_t)lds, st, k_start,
+                          k_stop, 0, a, groups, xq, xs, gather_src, act_q, act_s);
     return check_launch("gate_up_mfma");
 }
 

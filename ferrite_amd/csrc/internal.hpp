@@ -93,7 +93,7 @@ struct PackedLayout {
 PackedLayout packed_layout(const ferrite_moe_shape& s);
 int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
                         int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
-                        hipStream_t st);
+                        hipStream_t st, hipEvent_t k_start = nullptr, hipEvent_t k_stop = nullptr);
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
                      int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st);
 

@@ -272,7 +272,10 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     } else {
         uint8_t* act_q = reinterpret_cast<uint8_t*>(b + w.act);
         uint8_t* act_s = reinterpret_cast<uint8_t*>(b + w.act_s);
-        if ((rc = launch_gate_up_mfma(s, packed, xq, xs, n, gather_src, units, act_q, act_s, st))) return rc;
+        if ((rc = launch_gate_up_mfma(s, packed, xq, xs, n, gather_src, units, act_q, act_s, st,
+                                      ev ? static_cast<hipEvent_t>(ev[8]) : nullptr,
+                                      ev ? static_cast<hipEvent_t>(ev[9]) : nullptr)))
+            return rc;
         if ((rc = mark(ev, 5, st))) return rc;
         if ((rc = launch_down_mfma(s, packed, act_q, act_s, n, units, y, y_dtype, st))) return rc;
     }

@@ -232,8 +232,10 @@ int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_we
  * reference's FERRITE_TIMING probes (crates/ferrite-exec/src/lib.rs:1184-1299).  stage_events_host is a host
  * array of FERRITE_MOE_STAGE_EVENTS hipEvent_t handles (any may be NULL): [0] before the router GEMM, then
  * after: [1] router GEMM, [2] routing, [3] permutation, [4] activation quantisation (== [3] in f32 mode),
- * [5] gate/up GEMM + SwiGLU, [6] down GEMM, [7] combine.  Not capturable. */
-#define FERRITE_MOE_STAGE_EVENTS 8
+ * [5] gate/up GEMM + SwiGLU, [6] down GEMM, [7] combine; [8] and [9] bracket the gate/up kernel itself on the
+ * device (start and end of its execution, without the launch gap that [4]..[5] includes; MFMA mode only).
+ * Not capturable. */
+#define FERRITE_MOE_STAGE_EVENTS 10
 int ferrite_moe_layer_mxfp4_timed(const ferrite_moe_shape* shape, const ferrite_moe_weights* w,
                                   const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
                                   int out_dtype, int mode, void* workspace, size_t workspace_bytes,
