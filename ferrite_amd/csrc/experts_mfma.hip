@@ -431,6 +431,7 @@ struct PfCtx {
     const u4v* asp[2];        // weight scale words of the wave's two items
     const uint8_t* bsp[4];    // activation scale rows of the lane's column in the wave's 4 row tiles
     int KT, wave, wi, wt, lane, bslot;
+    int ntile;                // row tiles of this wave that hold rows of the unit (0..4): the others get no MFMAs
 };
 
 // Starts the loads of k step kt into `stage`.
@@ -473,15 +474,16 @@ __device__ __forceinline__ void pf_step(const PfCtx& c, u4v* lds, int kt, const 
     pf_fill(c, lds + ((Q + 1) & 1) * PF_LDS_STAGE, min(kt + 1, c.KT - 1));
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int ii = 0; ii < 2; ++ii) {
-        const uint32_t scs[4] = {asc[ii][0], asc[ii][1], asc[ii][2], asc[ii][3]};
+    for (int tt = 0; tt < 4; ++tt) {
+        if (tt >= c.ntile) break;   // wave-uniform: a unit's last block of rows is usually far from full
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const v8i a8 = {(int)av[ii][t][0], (int)av[ii][t][1], (int)av[ii][t][2], (int)av[ii][t][3], 0, 0, 0, 0};
+        for (int ii = 0; ii < 2; ++ii) {
 #pragma unroll
-            for (int tt = 0; tt < 4; ++tt)
+            for (int t = 0; t < 4; ++t) {
+                const v8i a8 = {(int)av[ii][t][0], (int)av[ii][t][1], (int)av[ii][t][2], (int)av[ii][t][3], 0, 0, 0, 0};
                 acc[ii][t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    a8, bv[tt], acc[ii][t][tt], 4 /*A e2m1*/, 0 /*B e4m3*/, Q, (int)scs[t], Q, (int)bsc[tt]);
+                    a8, bv[tt], acc[ii][t][tt], 4 /*A e2m1*/, 0 /*B e4m3*/, Q, (int)asc[ii][t], Q, (int)bsc[tt]);
+            }
         }
     }
     __builtin_amdgcn_sched_barrier(0);   // the MFMAs stay in front of the wait: they are what hides the loads
@@ -541,6 +543,7 @@ __device__ __forceinline__ void pf_context(PfCtx& c, const uint8_t* cbase, const
     c.lane = threadIdx.x & 63;
     c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     c.wi = c.wave % (PF_ITEMS / 2); c.wt = c.wave / (PF_ITEMS / 2);
+    c.ntile = min(4, max(0, (nrows - c.wt * 64 + 15) >> 4));
     const int cc = c.lane & 15, g = c.lane >> 4;
     c.a_src = reinterpret_cast<const u4v*>(cbase) + (size_t)min(item0 + c.wave, items - 1) * KT * 256 + c.lane;
     // Activation stage layout: the four lanes of a quad fetch 64 consecutive bytes of one row (what the texture
