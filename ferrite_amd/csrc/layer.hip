@@ -214,7 +214,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     if (fused_head) {
         // 1-3 (+ activation quantisation) as one launch
         PackedLayout L = packed_layout(s);
-        const int fuse_perm = n <= 64;
+        const int fuse_perm = 1;   // the block that routes the last token builds the tables
         if ((rc = launch_moe_head(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), wts->router_bias, s,
                                   n, logits, probs, ids_f32, ids, xq, xs, reinterpret_cast<int32_t*>(b + w.counters),
                                   reinterpret_cast<int32_t*>(b + w.counts), reinterpret_cast<int32_t*>(b + w.starts),

@@ -551,7 +551,7 @@ struct HeadArgs {
     int32_t* ids;
     uint8_t *xq, *xs;     // may be NULL: no quantisation blocks are launched then
     int32_t* counters;    // [1 + n]
-    int fuse_perm;        // the last routed token also builds the permutation (small n); else a separate launch does
+    int fuse_perm;        // the block that routes the last token also builds the permutation; else a separate launch does
     PermArgs perm;
 };
 
@@ -692,6 +692,20 @@ __device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const floa
     }
 }
 
+// The barriers of head_producer / head_consumer and nothing else.
+template <int T, int W>
+__device__ __forceinline__ void head_bystander(int nk4) {
+    const int nch = nk4 / HeadCfg<T, W>::CH;
+    __syncthreads();
+    __syncthreads();
+    for (int c = 0; c < nch; c += 4) {
+        __syncthreads();
+        __syncthreads();
+        __syncthreads();
+        __syncthreads();
+    }
+}
+
 template <typename XT, bool kFused, int T, int W>
 __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
     extern __shared__ __align__(16) unsigned char head_lds[];
@@ -727,7 +741,8 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
         }
         xl[i] = v;
     }
-    // wave 0 chains; wave 4 would share its SIMD (and its VALU issue slots) and leaves; the others produce
+    // wave 0 chains; wave 4 would share its SIMD (and its VALU issue slots) and only keeps the barriers company; the
+    // others produce
     float s[T];
 #pragma unroll
     for (int ti = 0; ti < T; ++ti) s[ti] = 0.0f;
@@ -739,39 +754,50 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
         case 5: head_producer<T, W, 3>(wp, a.Epad, nk4, xl, ring, lane); break;
         case 6: head_producer<T, W, 4>(wp, a.Epad, nk4, xl, ring, lane); break;
         case 7: head_producer<T, W, 5>(wp, a.Epad, nk4, xl, ring, lane); break;
-        default: __syncthreads(); break;   // its share of x is in LDS before it goes
+        default: head_bystander<T, W>(nk4); break;
     }
-    if (wave != 0) return;   // from here on the block is wave 0 alone; LDS is free for the scratch below
-    const int e = eb * 64 + lane;
+    // From here on wave 0 works alone (LDS is free for its scratch); with a fused permutation the other waves wait
+    // at the barrier below and join in if this block turns out to be the one that routed the last token.
+    const bool block_perm = kFused && a.fuse_perm;
+    if (wave != 0 && !block_perm) return;
+    __shared__ int perm_here;
+    int do_perm = 0;
+    if (wave == 0) {
+        const int e = eb * 64 + lane;
 #pragma unroll
-    for (int ti = 0; ti < T; ++ti) {
-        const int t = t0 + ti;
-        if (t >= a.n) break;
-        if (e < a.E) a.logits[(size_t)t * a.E + e] = s[ti];
-        if constexpr (kFused) {
-            // arrival: the stores above are made visible before the counter moves
-            __threadfence();
-            int last = 0;
-            if (lane == 0) last = atomicAdd(&a.counters[1 + t], 1) == eblocks - 1;
-            last = __shfl(last, 0, 64);
-            if (!last) continue;
-            __threadfence();
-            wave_sync();
-            RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds);
-            route_wave<true>(a.logits + (size_t)t * a.E, a.bias, true, a.E, a.topk, a.n_group, a.topk_group, a.scaling,
-                             sc, a.probs + (size_t)t * a.topk, a.ids_f32 + (size_t)t * a.topk,
-                             a.ids + (size_t)t * a.topk);
-            __threadfence();
-            last = 0;
-            if (lane == 0) last = atomicAdd(&a.counters[0], 1) == a.n - 1;
-            last = __shfl(last, 0, 64);
-            if (!last) continue;
-            __threadfence();
-            wave_sync();
-            if (a.fuse_perm) permute_in_block<true, true>(a.perm, reinterpret_cast<unsigned long long*>(head_lds));
-            for (int i = lane; i < a.n + 1; i += 64) a.counters[i] = 0;
+        for (int ti = 0; ti < T; ++ti) {
+            const int t = t0 + ti;
+            if (t >= a.n) break;
+            if (e < a.E) a.logits[(size_t)t * a.E + e] = s[ti];
+            if constexpr (kFused) {
+                // arrival: the stores above are made visible before the counter moves
+                __threadfence();
+                int last = 0;
+                if (lane == 0) last = atomicAdd(&a.counters[1 + t], 1) == eblocks - 1;
+                last = __shfl(last, 0, 64);
+                if (!last) continue;
+                __threadfence();
+                wave_sync();
+                RouteScratch& sc = *reinterpret_cast<RouteScratch*>(head_lds);
+                route_wave<true>(a.logits + (size_t)t * a.E, a.bias, true, a.E, a.topk, a.n_group, a.topk_group,
+                                 a.scaling, sc, a.probs + (size_t)t * a.topk, a.ids_f32 + (size_t)t * a.topk,
+                                 a.ids + (size_t)t * a.topk);
+                __threadfence();
+                last = 0;
+                if (lane == 0) last = atomicAdd(&a.counters[0], 1) == a.n - 1;
+                last = __shfl(last, 0, 64);
+                if (!last) continue;
+                __threadfence();
+                wave_sync();
+                do_perm = 1;
+                for (int i = lane; i < a.n + 1; i += 64) a.counters[i] = 0;
+            }
         }
+        if (lane == 0) perm_here = do_perm;
     }
+    if (!block_perm) return;
+    __syncthreads();
+    if (perm_here) permute_in_block<true, false>(a.perm, reinterpret_cast<unsigned long long*>(head_lds));
 }
 
 // tokens per block: two when one per block would not fit the chip's 256 CUs in one round
@@ -796,7 +822,7 @@ static size_t head_lds_bytes(int n, int H, int E, bool fused) {
 }
 
 bool head_supported(int n, int H, int E) {
-    return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, H, E, true) <= 160 * 1024;
+    return n <= HEAD_MAX_N && E <= RT_MAX_E && (H % 128) == 0 && head_lds_bytes(n, H, E, true) <= 160 * 1024 - 64;   // 64: the kernel's static LDS
 }
 
 template <typename XT, bool kFused, int T, int W>
