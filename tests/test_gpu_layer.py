@@ -209,7 +209,8 @@ def test_layer_fused_head_shapes(hip, oracle, n, e, bf16):
     """The fused routing kernel picks its block shape from n x (blocks of 64 experts): one token per block with a
     wide product ring (up to 256 blocks), one token with a narrow ring so that two blocks share a CU (up to 512),
     two tokens per block beyond that.  Logits, routing and tables are bit-exact in each, for f32 and bf16 input,
-    with n odd against the two-token blocks and the separate permutation launch (n > 64)."""
+    with n odd against the two-token blocks, and above 64 tokens, where the permutation that the last block builds
+    spans several 64-token chunks."""
     cfg = synth.MoeConfig(n, 384, e, 4, 128, 128, 4, 2, act_bf16=bf16)
     inp = synth.make_inputs(cfg, seed=23)
     layer = hip.load_moe_layer(inp)
