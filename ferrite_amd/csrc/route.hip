@@ -678,6 +678,7 @@ __device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const floa
     const int nch = nk4 / CH;
     const float4* b0 = ring;
     const float4* b1 = ring + CH * T * 64;
+    __builtin_amdgcn_s_setprio(3);   // ahead of another block's producer waves on the same SIMD
     __syncthreads();
     __syncthreads();
     for (int c = 0; c < nch; c += 4) {
@@ -690,6 +691,7 @@ __device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const floa
         if (c + 3 < nch) head_consume<T, W>(s, b1, lane);
         __syncthreads();
     }
+    __builtin_amdgcn_s_setprio(0);
 }
 
 // The barriers of head_producer / head_consumer and nothing else.
