@@ -490,10 +490,17 @@ __global__ __launch_bounds__(512) void permute_scan_kernel(PermArgs a, const uns
     const int nchunk = (a.n + 63) >> 6;
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         int run = 0;
-        for (int c = 0; c < nchunk; ++c) {
-            goffs[(size_t)e * nchunk + c] = run;
-            run += __popcll(gmask[(size_t)e * nchunk + c]);
+        const unsigned long long* me = gmask + (size_t)e * nchunk;
+        int32_t* oe = goffs + (size_t)e * nchunk;
+        int c = 0;
+        for (; c + 8 <= nchunk; c += 8) {   // eight loads in flight: the walk is memory latency
+            unsigned long long m[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) m[j] = me[c + j];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { oe[c + j] = run; run += __popcll(m[j]); }
         }
+        for (; c < nchunk; ++c) { oe[c] = run; run += __popcll(me[c]); }
         cnt[e] = run;
     }
     __syncthreads();
@@ -533,9 +540,9 @@ __global__ __launch_bounds__(256) void permute_scatter_kernel(PermArgs a, const 
 //                                  (two interleaved chains in wave 0, the weights fetched once for both)
 //   blocks (eblocks, t)          : e4m3-per-32 quantisation of x[t] (off the critical path)
 //   last logits block of a token : its wave 0 routes the token (arrival counter per token)
-//   last routed token            : builds the permutation and unit tables (up to 64 tokens; above that one wave
-//                                  is too slow for it and a separate launch follows), then clears the counters
-//                                  so the next launch (or graph replay) starts clean
+//   last routed token            : its block builds the permutation and unit tables with all of its waves (the
+//                                  others have been waiting at a barrier for the chain wave's verdict) and clears
+//                                  the counters so the next launch (or graph replay) starts clean
 // counters[0] = routed tokens, counters[1 + t] = logits blocks of token t that have arrived; all zero on entry.
 // ------------------------------------------------------------------------------------------------
 constexpr int HEAD_MAX_N = 256;
