@@ -1017,7 +1017,7 @@ int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n
         if (x_dtype == FERRITE_DT_BF16) return launch_router_tile<uint16_t>(x, router_t, n, H, E, logits, st);
         return FERRITE_ERR_INVALID_ARG;
     }
-    if (head_lds_bytes(n, H, E, false) > 160 * 1024) return FERRITE_DECLINED;
+    if (head_lds_bytes(n, H, E, false) > 160 * 1024 - 64) return FERRITE_DECLINED;   // 64: the kernel's static LDS
     HeadArgs a{};
     a.x = x; a.wt = router_t; a.n = n; a.H = H; a.E = E; a.Epad = (E + 63) / 64 * 64; a.logits = logits;
     const size_t lds = head_lds_bytes(n, H, E, false);
