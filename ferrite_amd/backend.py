@@ -24,11 +24,12 @@ from .synth import MoeConfig, MoeInputs
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 DEFAULT_SO = os.path.join(_HERE, "libferrite_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 OK, ERR_INVALID_ARG, DECLINED, ERR_WORKSPACE, ERR_RUNTIME = 0, 1, 2, 3, 4
 DT_F32, DT_BF16 = 0, 1
 MODE_F32_CHECK, MODE_MFMA_FP8 = 0, 1
+OVERRIDE_UNIT_ROWS, OVERRIDE_Y_F32 = 0, 1
 
 
 class FerriteError(RuntimeError):
@@ -80,7 +81,8 @@ class WorkspaceView(C.Structure):
 
 
 EXPORTS = [
-    "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_matmul_f32", "ferrite_rmsnorm_f32", "ferrite_hc_post_f32",
+    "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_hip_warmup",
+    "ferrite_hip_set_override", "ferrite_matmul_f32", "ferrite_rmsnorm_f32", "ferrite_hc_post_f32",
     "ferrite_swiglu_limited_f32", "ferrite_moe_route", "ferrite_moe_permute_scratch_bytes", "ferrite_moe_permute",
     "ferrite_mxfp4_dequant", "ferrite_mxfp4_quant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes",
     "ferrite_moe_pack_weights", "ferrite_moe_pack_expert", "ferrite_moe_pack_router",
@@ -106,7 +108,9 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_hc_post_f32.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, vp]
     lib.ferrite_moe_route.argtypes = [vp, vp, i32, i32, i32, i32, i32, f32, vp, vp, vp, vp]
     lib.ferrite_moe_permute_scratch_bytes.restype = sz
-    lib.ferrite_moe_permute_scratch_bytes.argtypes = [i32, i32]
+    lib.ferrite_moe_permute_scratch_bytes.argtypes = [i32, i32, i32]
+    lib.ferrite_hip_warmup.argtypes = []
+    lib.ferrite_hip_set_override.argtypes = [i32, i32]
     lib.ferrite_moe_permute.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     lib.ferrite_mxfp4_dequant.argtypes = [vp, vp, i64, i64, vp, vp]
     lib.ferrite_act_quant_fp8.argtypes = [vp, i32, i64, i32, vp, vp, vp]
@@ -230,6 +234,8 @@ class HipBackend:
         self._capturing = False
         self._graphs: Dict[str, int] = {}
         self._verify_ok = False
+        self._overrides = {OVERRIDE_UNIT_ROWS: 0, OVERRIDE_Y_F32: 0}
+        self._ck(self.lib.ferrite_hip_warmup(), "warmup")   # LDS limits, before any capture (cuda.rs:627-657)
 
     # ---- plumbing ----
     @property
@@ -270,6 +276,12 @@ class HipBackend:
 
     def sync(self):
         self.stream.synchronize()
+
+    def set_override(self, which: int, value: int):
+        """Process-wide test hook of the library (token tile of the expert GEMMs, f32 expert outputs).  Changes the
+        workspace layout: cached workspaces of a layer must be dropped by the caller (layer._ws.clear())."""
+        self._ck(self.lib.ferrite_hip_set_override(which, value), "set_override")
+        self._overrides[which] = value
 
     def upload(self, a, dtype=None) -> torch.Tensor:
         t = torch.from_numpy(np.ascontiguousarray(a))
@@ -381,7 +393,7 @@ class HipBackend:
         mk = lambda m: torch.empty(m, dtype=torch.int32, device=self.device)
         t = dict(counts=mk(n_experts), starts=mk(n_experts + 1), perm_map=mk(n * topk), gather_src=mk(n * topk),
                  active=mk(n_experts), n_active=mk(1))
-        sb = self.lib.ferrite_moe_permute_scratch_bytes(n, n_experts)
+        sb = self.lib.ferrite_moe_permute_scratch_bytes(n, topk, n_experts)
         scratch = torch.empty(max(sb, 16), dtype=torch.uint8, device=self.device)
         self._enter()
         self._ck(self.lib.ferrite_moe_permute(ids.data_ptr(), n, topk, n_experts, t["counts"].data_ptr(),
@@ -593,7 +605,7 @@ class HipBackend:
 
         E, k = cfg.n_experts, cfg.topk
         y_bf16 = (mode == MODE_MFMA_FP8 and self.unit_rows(layer, n, mode) == 128
-                  and os.environ.get("FERRITE_HIP_Y_F32") != "1")
+                  and not self._overrides[OVERRIDE_Y_F32])
         y_dtype = torch.bfloat16 if y_bf16 else torch.float32
         return dict(logits=view(v.logits, n * E, torch.float32).view(n, E),
                     probs=view(v.probs, n * k, torch.float32).view(n, k),

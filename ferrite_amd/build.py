@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 SO_PATH = os.path.join(HERE, "libferrite_hip.so")
 SOURCES = ["layer.hip", "route.hip", "formats.hip", "experts_f32.hip", "experts_mfma.hip", "block_ops.hip"]
-HEADERS = ["internal.hpp", "numerics.hpp", "device_utils.hpp", "prefill_mainloop_asm.inc", "gen_prefill_asm.py"]
+HEADERS = ["internal.hpp", "numerics.hpp", "device_utils.hpp"]
 
 
 def source_hash() -> str:
@@ -29,27 +29,62 @@ def source_hash() -> str:
     return h.hexdigest()[:16]
 
 
-def build(verbose: bool = False) -> str:
-    """Compile every HIP source into libferrite_hip.so (always recompiles)."""
+def build(verbose: bool = False, incremental: bool = False) -> str:
+    """Compile every HIP source into libferrite_hip.so: one object per source, compiled side by side, then linked.
+    Always recompiles unless `incremental` is set, which keeps the objects whose inputs (the source, the shared
+    headers, the flags) have not changed since they were built - a convenience while editing one kernel file."""
+    from concurrent.futures import ThreadPoolExecutor
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     build_id = "ferrite-hip-" + source_hash()
-    cmd = [hipcc, "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC", "-shared",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           # a*b+c must stay two rounded operations: routing has to reproduce the reference's f32 chains bit
-           # for bit (HIP's __fmul_rn/__fadd_rn are plain operators and would otherwise be fused); fmaf() where
-           # a fused multiply-add is wanted is written explicitly
-           "-ffp-contract=off",
-           "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
-           f'-DFERRITE_BUILD_ID="{build_id}"', "-I", INCLUDE, "-o", SO_PATH]
-    cmd += [os.path.join(CSRC, s) for s in SOURCES]
+    flags = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             # a*b+c must stay two rounded operations: routing has to reproduce the reference's f32 chains bit
+             # for bit (HIP's __fmul_rn/__fadd_rn are plain operators and would otherwise be fused); fmaf() where
+             # a fused multiply-add is wanted is written explicitly
+             "-ffp-contract=off",
+             "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes", "-I", INCLUDE]
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    shared = hashlib.sha256(" ".join(flags).encode())
+    for name in HEADERS:
+        with open(os.path.join(CSRC, name), "rb") as f:
+            shared.update(f.read())
+    with open(os.path.join(INCLUDE, "ferrite_hip.h"), "rb") as f:
+        shared.update(f.read())
+
+    def compile_one(src: str):
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        with open(os.path.join(CSRC, src), "rb") as f:
+            key = hashlib.sha256(shared.digest() + f.read()).hexdigest()
+        # the build id is baked into layer.hip only, so the other objects do not depend on it
+        extra = [f'-DFERRITE_BUILD_ID="{build_id}"'] if src == "layer.hip" else []
+        if src == "layer.hip":
+            key = hashlib.sha256((key + build_id).encode()).hexdigest()
+        stamp = obj + ".key"
+        if incremental and os.path.exists(obj) and os.path.exists(stamp) and open(stamp).read() == key:
+            return obj, ""
+        cmd = [hipcc] + flags + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd))
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            sys.stderr.write(res.stdout + res.stderr)
+            raise RuntimeError(f"hipcc failed on {src}")
+        with open(stamp, "w") as f:
+            f.write(key)
+        return obj, res.stderr
+
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 1)) as pool:
+        results = list(pool.map(compile_one, SOURCES))
     if verbose:
-        print(" ".join(cmd))
+        for _, err in results:
+            if err:
+                sys.stderr.write(err)
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", SO_PATH] + [o for o, _ in results]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
-        raise RuntimeError("hipcc failed")
-    if verbose and res.stderr:
-        sys.stderr.write(res.stderr)
+        raise RuntimeError("hipcc link failed")
     return SO_PATH
 
 
@@ -80,5 +115,5 @@ def build_host(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose="-v" in sys.argv, incremental="--incremental" in sys.argv))
     print(build_host(verbose=True))

@@ -35,8 +35,10 @@ __device__ __forceinline__ uint32_t e4m3_encode4_hw(float a, float b, float c, f
 // Clamped SwiGLU (cpu.rs:192-201) for the MFMA mode, whose results are rounded to e4m3 right afterwards: the
 // hardware exponential and reciprocal (a few ulp) instead of the bit-exact expf and division of swiglu_ref().
 __device__ __forceinline__ float swiglu_fast(float g, float u, float limit) {
-    const float gi = fminf(g, limit);
-    const float ui = fminf(fmaxf(u, -limit), limit);
+    // compare-and-select like swiglu_ref (cpu.rs:192-201), not fminf / fmaxf: those return the non-NaN operand and
+    // would turn a NaN accumulator into +-limit
+    const float gi = g > limit ? limit : g;
+    const float ui = u < -limit ? -limit : (u > limit ? limit : u);
     return gi * __builtin_amdgcn_rcpf(1.0f + __expf(-gi)) * ui;
 }
 

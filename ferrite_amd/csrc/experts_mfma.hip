@@ -415,7 +415,6 @@ constexpr int PF_WAVES = PF_ITEMS;                     // one wave per item for 
 constexpr int PF_A_SLOTS = PF_ITEMS * 256;             // u4v of weights per stage
 constexpr int PF_LDS_STAGE = PF_A_SLOTS + 1024;        // + 1024 activation slots
 constexpr size_t PF_LDS_BYTES = 2 * PF_LDS_STAGE * 16;  // 64 KiB (4 items) / 96 KiB (8 items)
-constexpr int PR_ITEMS = 4;
 
 typedef __attribute__((address_space(3))) void lds_void;
 typedef const __attribute__((address_space(1))) void glb_void;
@@ -684,213 +683,10 @@ __global__ __launch_bounds__(PF_WAVES * 64, PF_WAVES == 4 ? 2 : 1) void down_pre
     }
 }
 
-// ---- prefill kernels with the main loop in assembly ("pr") --------------------------------------------------
-// What bounds the kernels above is the latency of their global -> LDS fills: a block has one 32 KiB stage in flight,
-// 64 KiB per CU, and a stage takes about 1.6 us to land while the MFMAs of a k step take 0.43 us.  A deeper ring
-// cannot be expressed in C++: with a global -> LDS load in flight the compiler turns every wait it inserts into a
-// wait for everything, and it copies the results of asynchronous inline-assembly loads before they have arrived.
-// So the loop is one assembly block with fixed registers (prefill_mainloop_asm.inc, generated by
-// gen_prefill_asm.py): only the activations go through LDS, in a ring of six 16 KiB stages (four in flight); every
-// wave streams the weights of its own item from global memory into registers two pairs of k steps ahead, as the
-// 16-row kernels do.  One block = 4 waves = 4 items x one 128-row unit; wave w computes item w against all 8 row
-// tiles: 32 MFMAs per k step on 128 accumulators (a[0:127]), one block per CU.  A k step:
-//   reads of row tiles 4-7 (stage kt) | fill for step kt+5, on even steps the weights of the pair after next |
-//   16 MFMAs on row tiles 0-3 | wait: own reads, own quarter of stage kt+1; barrier | reads of row tiles 0-3 of
-//   stage kt+1 | 16 MFMAs on row tiles 4-7 | wait for those reads.
-// The waits are counted: loads complete in issue order and every step issues a fixed number of them.  The k order
-// is that of the other kernels: same bits.  Needs K a multiple of 512.
-#include "prefill_mainloop_asm.inc"
-
-constexpr int PR_NS = 6;
-constexpr int PR_STAGE_BYTES = 16384;   // 8 row tiles x 2 halves x 64 lanes x 16 B
-
-static inline size_t pr_lds_bytes(int K) { return (size_t)PR_NS * PR_STAGE_BYTES + (size_t)(K / 512) * 2048; }
-
-template <int IDX>
-__device__ __forceinline__ float pr_acc() {
-    float v;
-    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(v) : "n"(IDX));
-    return v;
-}
-// accumulator tile (weight tile T, row tile TT): element v = (weight row 4*(lane/16) + v, unit column lane%16)
-template <int T, int TT>
-__device__ __forceinline__ v4f pr_acc_tile() {
-    constexpr int B = (T * 8 + TT) * 4;
-    return (v4f){pr_acc<B>(), pr_acc<B + 1>(), pr_acc<B + 2>(), pr_acc<B + 3>()};
-}
-
-// Runs the whole reduction; on return the accumulators are in a[0:127].  bbase: the buffer all activation rows
-// live in (their offsets from it fit 32 bits); row_q(col) / row_s(col): the e4m3 row and the scale row (operand
-// order) of unit column col < nrows.
-template <typename RowQ, typename RowS>
-__device__ __forceinline__ void pr_mainloop(unsigned char* lds, const uint8_t* cbase, const uint8_t* sbase, int item,
-                                            int KT, int nrows, const uint8_t* bbase, RowQ row_q, RowS row_s) {
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int cc = lane & 15, g = lane >> 4, KT4 = KT >> 2;
-    // activation scale words of the whole unit into LDS: [group][row tile][lane] (ordinary stores, before any fill)
-    {
-        uint32_t* scl = reinterpret_cast<uint32_t*>(lds + PR_NS * PR_STAGE_BYTES);
-        for (int idx = threadIdx.x; idx < KT4 * 512; idx += 256) {
-            const int l = idx & 63, tt = (idx >> 6) & 7, k4 = idx >> 9;
-            const int col = tt * 16 + (l & 15);
-            scl[idx] = *reinterpret_cast<const uint32_t*>(row_s(col < nrows ? col : 0) + k4 * 16 + (l >> 4) * 4);
-        }
-    }
-    __syncthreads();
-    const uint8_t* wbase = cbase + (size_t)item * KT * 4096;
-    const uint8_t* wsbase = sbase + (size_t)item * KT4 * 1024;
-    uint32_t wo0 = (uint32_t)lane * 16, wo1 = wo0 + 4096, wso = wo0;
-    // staging layout of the activations as in the kernels above: quad-contiguous, XOR-slotted
-    uint32_t bo[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int col = (wave * 2 + i) * 16 + (lane >> 2);
-        const uint32_t o = (uint32_t)(row_q(col < nrows ? col : 0) - bbase) + ((lane & 3) ^ ((lane >> 3) & 3)) * 16;
-        bo[i][0] = o;
-        bo[i][1] = o + 64;
-    }
-    const uint32_t ring = (uint32_t)(uintptr_t)(lds_void*)lds;   // the 32-bit LDS address of the generic pointer
-    const uint32_t rd0 = ring + (uint32_t)(4 * cc + (g ^ ((cc >> 1) & 3))) * 16, rd1 = rd0 + 65536;
-    uint32_t sc = ring + PR_NS * PR_STAGE_BYTES + (uint32_t)lane * 4;
-    const uint32_t ldsw = ring + (uint32_t)wave * 4096;
-    int nfill = KT - 1, npair = (KT >> 1) - 1, nsc = KT4 - 1, grp = KT4;
-    uint32_t t0, t1;
-    asm volatile(PR_MAINLOOP_ASM
-                 : [wo0] "+v"(wo0), [wo1] "+v"(wo1), [wso] "+v"(wso), [bo0] "+v"(bo[0][0]), [bo1] "+v"(bo[0][1]),
-                   [bo2] "+v"(bo[1][0]), [bo3] "+v"(bo[1][1]), [sc] "+v"(sc), [nfill] "+s"(nfill), [npair] "+s"(npair),
-                   [nsc] "+s"(nsc), [grp] "+s"(grp), [t0] "=&s"(t0), [t1] "=&s"(t1)
-                 : [wbase] "s"(wbase), [wsbase] "s"(wsbase), [bbase] "s"(bbase), [rd0] "v"(rd0), [rd1] "v"(rd1),
-                   [ldsw] "s"(ldsw)
-                 : PR_MAINLOOP_CLOBBERS);
-}
-
-template <int TT>
-__device__ __forceinline__ void pr_gate_up_store(const MfmaArgs& a, int row0, int nrows, int item, int lane,
-                                                 uint8_t* __restrict__ act_q, uint8_t* __restrict__ act_s) {
-    // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
-    const int cc = lane & 15, g = lane >> 4, col = TT * 16 + cc;
-    const v4f g0 = pr_acc_tile<0, TT>(), g1 = pr_acc_tile<1, TT>(), u0 = pr_acc_tile<2, TT>(), u1 = pr_acc_tile<3, TT>();
-    float r0[4], r1[4];
-    float amax = 0.0f;
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        r0[v] = swiglu_fast(g0[v], u0[v], a.limit);
-        r1[v] = swiglu_fast(g1[v], u1[v], a.limit);
-        amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
-    }
-    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-    if (col < nrows) {
-        const uint32_t sb = block_scale_e8m0(amax);
-        const float inv = u2f((254u - sb) << 23);
-        const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
-        const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
-        uint8_t* dst = act_q + (size_t)(row0 + col) * a.act_ld + (size_t)item * 32 + g * 4;
-        *reinterpret_cast<uint32_t*>(dst) = p0;
-        *reinterpret_cast<uint32_t*>(dst + 16) = p1;
-        if (g == 0) act_s[(size_t)(row0 + col) * scale_pitch(a.act_ld) + scale_pos(item)] = (uint8_t)sb;
-    }
-}
-
-__global__ __launch_bounds__(256, 1) void gate_up_pr_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
-                                                          const uint8_t* __restrict__ xs,
-                                                          const int32_t* __restrict__ gather_src,
-                                                          uint8_t* __restrict__ act_q, uint8_t* __restrict__ act_s) {
-    extern __shared__ __align__(16) unsigned char lds_raw[];
-    int u, ig, ne;
-    if (!unit_block_work(a, groups, u, ig, ne)) return;
-    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
-    if (!unit_ok(a, e, row0, nrows)) return;
-    const bool shared = e == a.n_experts;
-    const int inter = shared ? a.shared_inter : a.inter;
-    const int items = inter / 32, item0 = ig * PR_ITEMS;
-    if (item0 >= items) return;
-    const int H = a.hidden, nk = a.n * a.topk, topk = a.topk, n = a.n;
-    const int spitch = scale_pitch(H);
-    auto token = [&](int col) -> int {
-        const int gr = row0 + col;
-        if (shared) return gr - nk;
-        const int i = gather_src[gr];
-        const int tk = (i < 0 || i >= nk) ? 0 : i / topk;
-        return tk < n ? tk : 0;
-    };
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int item = item0 + wave;
-    pr_mainloop(lds_raw, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
-                shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), H / 128, nrows,
-                xq, [&](int col) { return xq + (size_t)token(col) * H; },
-                [&](int col) { return xs + (size_t)token(col) * spitch; });
-    if (item >= items) return;
-    pr_gate_up_store<0>(a, row0, nrows, item, lane, act_q, act_s);
-    pr_gate_up_store<1>(a, row0, nrows, item, lane, act_q, act_s);
-    pr_gate_up_store<2>(a, row0, nrows, item, lane, act_q, act_s);
-    pr_gate_up_store<3>(a, row0, nrows, item, lane, act_q, act_s);
-    pr_gate_up_store<4>(a, row0, nrows, item, lane, act_q, act_s);
-    pr_gate_up_store<5>(a, row0, nrows, item, lane, act_q, act_s);
-    pr_gate_up_store<6>(a, row0, nrows, item, lane, act_q, act_s);
-    pr_gate_up_store<7>(a, row0, nrows, item, lane, act_q, act_s);
-}
-
-template <typename YT, int TT>
-__device__ __forceinline__ void pr_down_store(int H, int row0, int nrows, int item, int lane, YT* __restrict__ y) {
-    const int cc = lane & 15, g = lane >> 4, col = TT * 16 + cc;
-    const v4f r[4] = {pr_acc_tile<0, TT>(), pr_acc_tile<1, TT>(), pr_acc_tile<2, TT>(), pr_acc_tile<3, TT>()};
-    if (col < nrows) {
-        YT* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            if constexpr (sizeof(YT) == 4)
-                *reinterpret_cast<float4*>(dst + t * 16) = make_float4(r[t][0], r[t][1], r[t][2], r[t][3]);
-            else
-                *reinterpret_cast<uint2*>(dst + t * 16) = make_uint2(bf16_rne(r[t][0]) | (bf16_rne(r[t][1]) << 16),
-                                                                     bf16_rne(r[t][2]) | (bf16_rne(r[t][3]) << 16));
-        }
-    }
-}
-
-template <typename YT>
-__global__ __launch_bounds__(256, 1) void down_pr_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
-                                                       const uint8_t* __restrict__ act_s, YT* __restrict__ y) {
-    extern __shared__ __align__(16) unsigned char lds_raw[];
-    int u, ig, ne;
-    if (!unit_block_work(a, groups, u, ig, ne)) return;
-    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
-    if (!unit_ok(a, e, row0, nrows)) return;
-    const bool shared = e == a.n_experts;
-    const int inter = shared ? a.shared_inter : a.inter;
-    const int H = a.hidden, items = H / 64, item0 = ig * PR_ITEMS;
-    if (item0 >= items) return;
-    const int apitch = scale_pitch(a.act_ld), act_ld = a.act_ld;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int item = item0 + wave;
-    pr_mainloop(lds_raw, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
-                shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), inter / 128,
-                nrows, act_q, [&](int col) { return act_q + (size_t)(row0 + col) * act_ld; },
-                [&](int col) { return act_s + (size_t)(row0 + col) * apitch; });
-    if (item >= items) return;
-    pr_down_store<YT, 0>(H, row0, nrows, item, lane, y);
-    pr_down_store<YT, 1>(H, row0, nrows, item, lane, y);
-    pr_down_store<YT, 2>(H, row0, nrows, item, lane, y);
-    pr_down_store<YT, 3>(H, row0, nrows, item, lane, y);
-    pr_down_store<YT, 4>(H, row0, nrows, item, lane, y);
-    pr_down_store<YT, 5>(H, row0, nrows, item, lane, y);
-    pr_down_store<YT, 6>(H, row0, nrows, item, lane, y);
-    pr_down_store<YT, 7>(H, row0, nrows, item, lane, y);
-}
-
 // ---- launchers ----------------------------------------------------------------------------------------
 constexpr int GU_WAVES = 4;
 constexpr int DN_WAVES = 4;
 constexpr int DN_IPW = 2;
-
-// The kernels with the assembly main loop take reduction lengths that are whole groups of four k steps and whose
-// activation scale words fit next to the ring.  Opt-in for now: FERRITE_HIP_PREFILL=asm.
-static bool prefill_asm_loop(int K) {
-    if (K % 512 != 0 || pr_lds_bytes(K) > 160 * 1024) return false;
-    const char* v = getenv("FERRITE_HIP_PREFILL");
-    return v && !strcmp(v, "asm");
-}
 
 static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int n, const UnitTables& units, bool down) {
     PackedLayout L = packed_layout(s);
@@ -920,21 +716,9 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     MfmaArgs a = make_args(s, packed, n, units, false);
     const int imax = a.act_ld;
     if (units.unit_rows_cap == PF_ROWS) {
-        const bool asm_loop = prefill_asm_loop(s.hidden);
-        const int ipb = asm_loop ? PR_ITEMS : PF_ITEMS;   // items per block
-        const int groups = (imax / 32 + ipb - 1) / ipb;
+        const int groups = (imax / 32 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-        if (asm_loop) {
-            static size_t raised_pr = 0;
-            const size_t lds = pr_lds_bytes(s.hidden);
-            int rc = set_lds_limit(gate_up_pr_kernel, lds, &raised_pr);
-            if (rc) return rc;
-            hipExtLaunchKernelGGL(gate_up_pr_kernel, dim3(blocks), dim3(256), (uint32_t)lds, st, k_start, k_stop, 0, a, groups,
-                                  xq, xs, gather_src, act_q, act_s);
-            return check_launch("gate_up_pr");
-        }
-        static size_t raised_pf = 0;
-        int rc = set_lds_limit(gate_up_prefill_kernel, PF_LDS_BYTES, &raised_pf);
+        int rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES);
         if (rc) return rc;
         hipExtLaunchKernelGGL(gate_up_prefill_kernel, dim3(blocks), dim3(PF_WAVES * 64), (uint32_t)PF_LDS_BYTES, st, k_start,
                               k_stop, 0, a, groups, xq, xs, gather_src, act_q, act_s);
@@ -942,8 +726,7 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     }
     if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = (size_t)s.hidden * 16 + (size_t)((s.hidden / 128 + 3) / 4) * 256;
-    static size_t raised = 0;
-    int rc = set_lds_limit(gate_up_mfma_kernel<GU_WAVES>, lds, &raised);
+    int rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES>>::ensure(lds);
     if (rc) return rc;
     const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
     const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
@@ -956,41 +739,21 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ui
                      int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
     MfmaArgs a = make_args(s, packed, n, units, true);
     if (units.unit_rows_cap == PF_ROWS) {
-        // every expert of the launch must qualify: routed and shared intermediate sizes
-        const bool asm_loop = prefill_asm_loop(s.inter) && (s.shared_inter == 0 || prefill_asm_loop(s.shared_inter));
-        const int ipb = asm_loop ? PR_ITEMS : PF_ITEMS;
-        const int groups = (s.hidden / 64 + ipb - 1) / ipb;
+        const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-        if (asm_loop) {
-            const size_t lds = pr_lds_bytes(a.act_ld);
-            int rc;
-            if (y_dtype == FERRITE_DT_BF16) {
-                static size_t raised = 0;
-                if ((rc = set_lds_limit(down_pr_kernel<uint16_t>, lds, &raised))) return rc;
-                down_pr_kernel<uint16_t><<<blocks, 256, lds, st>>>(a, groups, act_q, act_s, static_cast<uint16_t*>(y));
-            } else {
-                static size_t raised = 0;
-                if ((rc = set_lds_limit(down_pr_kernel<float>, lds, &raised))) return rc;
-                down_pr_kernel<float><<<blocks, 256, lds, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
-            }
-            return check_launch("down_pr");
-        }
         int rc;
         if (y_dtype == FERRITE_DT_BF16) {
-            static size_t raised = 0;
-            if ((rc = set_lds_limit(down_prefill_kernel<uint16_t>, PF_LDS_BYTES, &raised))) return rc;
+            if ((rc = LdsLimit<&down_prefill_kernel<uint16_t>>::ensure(PF_LDS_BYTES))) return rc;
             down_prefill_kernel<uint16_t><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<uint16_t*>(y));
         } else {
-            static size_t raised = 0;
-            if ((rc = set_lds_limit(down_prefill_kernel<float>, PF_LDS_BYTES, &raised))) return rc;
+            if ((rc = LdsLimit<&down_prefill_kernel<float>>::ensure(PF_LDS_BYTES))) return rc;
             down_prefill_kernel<float><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
         }
         return check_launch("down_prefill");
     }
     if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = (size_t)a.act_ld * 16 + (size_t)((a.act_ld / 128 + 3) / 4) * 256;
-    static size_t raised = 0;
-    int rc = set_lds_limit(down_mfma_kernel<DN_WAVES, DN_IPW>, lds, &raised);
+    int rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW>>::ensure(lds);
     if (rc) return rc;
     const int items = s.hidden / 64;
     const int groups = (items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW);
@@ -998,6 +761,15 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ui
     if (y_dtype != FERRITE_DT_F32) return FERRITE_ERR_INVALID_ARG;
     down_mfma_kernel<DN_WAVES, DN_IPW><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
     return check_launch("down_mfma");
+}
+
+int warmup_experts_mfma() {
+    int rc;
+    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES))) return rc;
+    if ((rc = LdsLimit<&down_prefill_kernel<uint16_t>>::ensure(PF_LDS_BYTES))) return rc;
+    return LdsLimit<&down_prefill_kernel<float>>::ensure(PF_LDS_BYTES);
 }
 
 }  // namespace fe

@@ -1,6 +1,7 @@
 // Declarations shared between the translation units of libferrite_hip.so (not part of the public ABI).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -36,25 +37,38 @@ inline int max_units_for(int n, int topk, int n_experts, int has_shared, int uni
 }
 
 // Rows per unit for a layer call: 128-row units (both GEMM operands tiled through LDS) once the average expert
-// sees enough rows to fill them, 16-row units (weights streamed once per unit) below that.  The environment
-// variable FERRITE_HIP_UNIT_ROWS (16 or 128) overrides the choice; it is read at every call.
+// sees enough rows to fill them, 16-row units (weights streamed once per unit) below that.  A process-wide override
+// (ferrite_hip_set_override, a test hook) forces either; nothing here reads the environment.
 int unit_rows_for(int n, int topk, int n_experts);
 // Element type of the expert outputs `y` in the workspace: bf16 for 128-row units (prefill-sized batches, where the
-// y round trip through HBM is a tenth of the layer), f32 otherwise.  FERRITE_HIP_Y_F32=1 forces f32 (tests).
+// y round trip through HBM is a tenth of the layer), f32 otherwise.  The FERRITE_OVERRIDE_Y_F32 override forces f32.
 int y_dtype_for(int unit_rows);
 
-// Kernels that need more than 64 KiB of dynamic LDS must have the limit raised once (a function attribute,
-// not a stream operation).  `raised` remembers the largest value already set for that kernel.
-template <typename K>
-inline int set_lds_limit(K kernel, size_t bytes, size_t* raised) {
-    if (bytes <= 64 * 1024 || bytes <= *raised) return FERRITE_OK;
-    if (bytes > 160 * 1024) return FERRITE_DECLINED;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
-    *raised = bytes;
-    return FERRITE_OK;
-}
+// Kernels that need more than 64 KiB of dynamic LDS must have the limit raised once per device (a function
+// attribute, not a stream operation, and therefore not something to do inside a stream capture:
+// ferrite_hip_warmup() raises every kernel's limit to the most it can ever ask for).  LdsLimit<kernel>::ensure()
+// is the per-launch check: an atomic read on the fast path, a mutex around the attribute call otherwise.
+constexpr size_t kLdsCap = 160 * 1024;
+constexpr int kMaxDevices = 16;
+int current_device(int* dev);
+int raise_lds_limit(const void* kernel, size_t bytes, std::atomic<size_t>* raised);
+
+template <auto Kernel>
+struct LdsLimit {
+    static inline std::atomic<size_t> raised[kMaxDevices] = {};
+    static int ensure(size_t bytes) {
+        if (bytes <= 64 * 1024) return FERRITE_OK;
+        if (bytes > kLdsCap) return FERRITE_DECLINED;
+        int dev = 0;
+        if (int rc = current_device(&dev)) return rc;
+        if (bytes <= raised[dev].load(std::memory_order_acquire)) return FERRITE_OK;
+        return raise_lds_limit(reinterpret_cast<const void*>(Kernel), bytes, &raised[dev]);
+    }
+};
+
+// Per translation unit: raise the LDS limit of every kernel in it that may exceed 64 KiB (ferrite_hip_warmup).
+int warmup_route();
+int warmup_experts_mfma();
 
 // route.hip
 int launch_matmul_exact(const void* x, int x_dtype, const float* w, const float* bias, float* out, int n, int k,
@@ -63,6 +77,8 @@ int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* 
                    int32_t* perm_map, int32_t* gather_src, int32_t* active, int32_t* n_active, void* scratch,
                    size_t scratch_bytes, const UnitTables* units, int has_shared, hipStream_t st);
 
+int check_routing_params(int e, int topk, int n_group, int topk_group);
+size_t perm_scratch_bytes(int n_tokens, int n_experts);   // masks + offsets of the three-phase permutation
 bool head_supported(int n, int H, int E);
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
                     int n, float* logits, float* probs, float* ids_f32, int32_t* ids, uint8_t* xq, uint8_t* xs,

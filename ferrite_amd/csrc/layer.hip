@@ -5,6 +5,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "internal.hpp"
 
 #ifndef FERRITE_BUILD_ID
@@ -35,18 +38,36 @@ struct Workspace {
     int max_units, rows, unit_cap;
 };
 
+// Process-wide overrides (ferrite_hip_set_override): test hooks that replace what used to be environment reads.
+static std::atomic<int> g_override_unit_rows{0};   // 0 = automatic, else 16 or 128
+static std::atomic<int> g_override_y_f32{0};       // 1 = expert outputs stay f32 on the 128-row path
+
 int unit_rows_for(int n, int topk, int n_experts) {
-    if (const char* v = getenv("FERRITE_HIP_UNIT_ROWS")) {
-        if (!strcmp(v, "16")) return 16;
-        if (!strcmp(v, "128")) return 128;
-    }
+    const int forced = g_override_unit_rows.load(std::memory_order_relaxed);
+    if (forced == 16 || forced == 128) return forced;
     return (long)n * topk >= 48L * n_experts ? 128 : 16;
 }
 
 int y_dtype_for(int unit_rows) {
     if (unit_rows != 128) return FERRITE_DT_F32;
-    const char* v = getenv("FERRITE_HIP_Y_F32");
-    return (v && !strcmp(v, "1")) ? FERRITE_DT_F32 : FERRITE_DT_BF16;
+    return g_override_y_f32.load(std::memory_order_relaxed) ? FERRITE_DT_F32 : FERRITE_DT_BF16;
+}
+
+int current_device(int* dev) {
+    hipError_t e = hipGetDevice(dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (*dev < 0 || *dev >= kMaxDevices) return FERRITE_ERR_INVALID_ARG;
+    return FERRITE_OK;
+}
+
+int raise_lds_limit(const void* kernel, size_t bytes, std::atomic<size_t>* raised) {
+    static std::mutex mu;   // attribute and record change together
+    std::lock_guard<std::mutex> lock(mu);
+    if (bytes <= raised->load(std::memory_order_relaxed)) return FERRITE_OK;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
+    raised->store(bytes, std::memory_order_release);
+    return FERRITE_OK;
 }
 
 static size_t bump(size_t& off, size_t bytes) {
@@ -81,7 +102,7 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     w.unit_first = bump(off, (size_t)w.max_units * 4);
     w.unit_count = bump(off, (size_t)w.max_units * 4);
     w.n_units = bump(off, 4);
-    w.perm_scratch_bytes = ferrite_moe_permute_scratch_bytes(n, s.n_experts);
+    w.perm_scratch_bytes = perm_scratch_bytes(n, s.n_experts);
     w.perm_scratch = bump(off, w.perm_scratch_bytes);
     if (mode == FERRITE_MODE_MFMA_FP8) {
         w.xq = bump(off, (size_t)n * H);
@@ -105,8 +126,9 @@ static int check_shape(const ferrite_moe_shape* s, int n, int mode) {
     if (s->hidden % 32 || s->inter % 32 || s->shared_inter % 32) return FERRITE_ERR_INVALID_ARG;
     if (mode == FERRITE_MODE_MFMA_FP8 && (s->hidden % 128 || s->inter % 128 || s->shared_inter % 128))
         return FERRITE_DECLINED;
-    if ((long long)n * s->topk > 0x7fffffffLL / 2) return FERRITE_DECLINED;
-    return FERRITE_OK;
+    if (n > 65535) return FERRITE_DECLINED;   // token index on grid.y of several kernels: split the batch
+    // the routing kernels' own limits, for the fused head and the separate launches alike
+    return check_routing_params(s->n_experts, s->topk, s->n_group, s->topk_group);
 }
 
 }  // namespace fe
@@ -116,6 +138,26 @@ using namespace fe;
 extern "C" const char* ferrite_kernel_build_id(void) { return FERRITE_BUILD_ID; }
 extern "C" unsigned ferrite_kernel_abi_version(void) { return FERRITE_ABI_VERSION; }
 extern "C" const char* ferrite_hip_last_error(void) { return g_last_error; }
+
+extern "C" int ferrite_hip_set_override(int which, int value) {
+    if (which == FERRITE_OVERRIDE_UNIT_ROWS) {
+        if (value != 0 && value != 16 && value != 128) return FERRITE_ERR_INVALID_ARG;
+        g_override_unit_rows.store(value);
+        return FERRITE_OK;
+    }
+    if (which == FERRITE_OVERRIDE_Y_F32) {
+        if (value != 0 && value != 1) return FERRITE_ERR_INVALID_ARG;
+        g_override_y_f32.store(value);
+        return FERRITE_OK;
+    }
+    return FERRITE_ERR_INVALID_ARG;
+}
+
+extern "C" int ferrite_hip_warmup(void) {
+    int rc;
+    if ((rc = warmup_route())) return rc;
+    return warmup_experts_mfma();
+}
 
 extern "C" int ferrite_moe_layer_unit_rows(const ferrite_moe_shape* shape, int n, int mode) {
     if (check_shape(shape, n, mode)) return 0;

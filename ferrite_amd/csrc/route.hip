@@ -210,6 +210,10 @@ __device__ __forceinline__ void route_wave_ni(const float* __restrict__ lg, cons
         if (ok[i]) l = kCoherent ? load_coherent(lg + j) : lg[j];
         sg[i] = sigmoid_ref(l);
         ch[i] = ok[i] ? fadd(sg[i], bias ? bias[j] : 0.0f) : 0.0f;
+        // A NaN score (NaN logit or bias) is never selected, as in the reference's device router, whose arg-max
+        // comparisons are false for NaN (kernels/cuda/ferrite_kernels.cu:1233-1241); slots that no finite score
+        // can fill keep id -1 and weight 0 (ferrite_kernels.cu:1255-1270).  CpuBackend panics instead (cpu.rs:560).
+        if (ch[i] != ch[i]) ok[i] = false;
     }
     if (lane < RT_MAX_K) { sc.sel_id[lane] = -1; sc.sel_sig[lane] = 0.0f; }
 
@@ -836,8 +840,7 @@ bool head_supported(int n, int H, int E) {
 
 template <typename XT, bool kFused, int T, int W>
 static int launch_head_tt(const HeadArgs& a, int quant, size_t lds, hipStream_t st) {
-    static size_t raised = 0;
-    int rc = set_lds_limit(moe_head_kernel<XT, kFused, T, W>, lds, &raised);
+    int rc = LdsLimit<&moe_head_kernel<XT, kFused, T, W>>::ensure(lds);
     if (rc) return rc;
     dim3 grid(a.Epad / 64 + quant, (a.n + T - 1) / T);
     moe_head_kernel<XT, kFused, T, W><<<grid, 512, lds, st>>>(a);
@@ -877,6 +880,37 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
     if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, xq ? 1 : 0, lds, st);
     if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, true>(a, xq ? 1 : 0, lds, st);
     return FERRITE_ERR_INVALID_ARG;
+}
+
+// What every routing kernel here assumes of its parameters, for the stand-alone op and for the fused head alike:
+// argument errors first (the reference returns Err for them, cpu.rs:539-545), then the limits of these kernels
+// (LDS arrays of RT_MAX_E keys, RT_MAX_K selections, one lane per group) as FERRITE_DECLINED.
+int check_routing_params(int e, int topk, int n_group, int topk_group) {
+    if (e <= 0 || topk <= 0 || topk > e) return FERRITE_ERR_INVALID_ARG;
+    if (n_group > 1) {
+        if (e % n_group != 0 || topk_group < 1 || topk_group > n_group) return FERRITE_ERR_INVALID_ARG;
+        if (topk > topk_group * (e / n_group)) return FERRITE_ERR_INVALID_ARG;
+        if (n_group > 64) return FERRITE_DECLINED;
+    }
+    if (e > RT_MAX_E || topk > RT_MAX_K) return FERRITE_DECLINED;
+    return FERRITE_OK;
+}
+
+template <typename XT, bool kFused>
+static int warmup_head() {
+    const size_t cap = kLdsCap - 64;   // 64: the kernel's static LDS
+    int rc;
+    if ((rc = LdsLimit<&moe_head_kernel<XT, kFused, 1, 32>>::ensure(cap))) return rc;
+    if ((rc = LdsLimit<&moe_head_kernel<XT, kFused, 1, 16>>::ensure(cap))) return rc;
+    return LdsLimit<&moe_head_kernel<XT, kFused, 2, 32>>::ensure(cap);
+}
+
+int warmup_route() {
+    int rc;
+    if ((rc = warmup_head<float, true>())) return rc;
+    if ((rc = warmup_head<uint16_t, true>())) return rc;
+    if ((rc = warmup_head<float, false>())) return rc;
+    return warmup_head<uint16_t, false>();
 }
 
 // Router GEMM for many tokens: the same sequential chain (cpu.rs:82-122), register tiled.  A wave owns 64 experts
@@ -1056,7 +1090,7 @@ int launch_zero_i32(int32_t* p, int count, hipStream_t st) {
     return check_launch("zero_i32");
 }
 
-static size_t perm_scratch_bytes(int n, int n_experts) {
+size_t perm_scratch_bytes(int n, int n_experts) {
     size_t nchunk = ((size_t)n + 63) / 64;
     return (size_t)n_experts * nchunk * (8 + 4) + 64;
 }
@@ -1124,24 +1158,18 @@ extern "C" int ferrite_swiglu_limited_f32(const float* gate_up, float limit, flo
 extern "C" int ferrite_moe_route(const float* logits, const float* bias, int n, int e, int topk, int n_group,
                                  int topk_group, float routed_scaling, float* probs, float* ids_f32,
                                  int32_t* ids_i32, ferrite_stream_t stream) {
-    if (n < 0 || e <= 0 || topk <= 0 || topk > e || !logits || !probs) return FERRITE_ERR_INVALID_ARG;
-    if (n_group < 1) n_group = 1;
-    if (n_group > 1) {
-        if (e % n_group != 0 || topk_group < 1 || topk_group > n_group) return FERRITE_ERR_INVALID_ARG;
-        if (topk > topk_group * (e / n_group)) return FERRITE_ERR_INVALID_ARG;
-        if (n_group > 64) return FERRITE_DECLINED;
-        if (topk_group == n_group) n_group = 1;  // keeps every expert: the ungrouped router
-    }
-    if (e > RT_MAX_E || topk > RT_MAX_K) return FERRITE_DECLINED;
+    if (n < 0 || !logits || !probs) return FERRITE_ERR_INVALID_ARG;
+    if (int rc = check_routing_params(e, topk, n_group, topk_group)) return rc;
+    if (n_group < 1 || topk_group == n_group) n_group = 1;  // keeps every expert: the ungrouped router
     if (n == 0) return FERRITE_OK;
     moe_route_kernel<<<(n + 3) / 4, 256, 0, as_stream(stream)>>>(logits, bias, n, e, topk, n_group, topk_group,
                                                                  routed_scaling, probs, ids_f32, ids_i32);
     return check_launch("moe_route");
 }
 
-extern "C" size_t ferrite_moe_permute_scratch_bytes(int n, int n_experts) {
-    if (n <= 0 || n_experts <= 0) return 0;
-    return perm_scratch_bytes(n, n_experts);
+extern "C" size_t ferrite_moe_permute_scratch_bytes(int n, int topk, int n_experts) {
+    if (n <= 0 || topk <= 0 || n_experts <= 0 || (long long)n * topk > 0x3fffffffLL) return 0;
+    return perm_scratch_bytes(n * topk, n_experts);
 }
 
 extern "C" int ferrite_moe_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* counts,
@@ -1149,6 +1177,11 @@ extern "C" int ferrite_moe_permute(const int32_t* ids, int n, int topk, int n_ex
                                    int32_t* n_active, void* scratch, size_t scratch_bytes,
                                    ferrite_stream_t stream) {
     if (!ids || !counts || !starts || !perm_map || !gather_src) return FERRITE_ERR_INVALID_ARG;
-    return launch_permute(ids, n, topk, n_experts, counts, starts, perm_map, gather_src, active, n_active, scratch,
+    if (n <= 0 || topk <= 0 || (long long)n * topk > 0x3fffffffLL) return FERRITE_ERR_INVALID_ARG;
+    // The kernels rank an assignment by the earlier *tokens* that chose its expert, which is right when a token
+    // holds each expert at most once (what a router emits).  This stand-alone op promises nothing about its ids
+    // (the reference's own vector, chain_dev.rs:25042, lists an expert twice in one token), so it runs them with
+    // every assignment as a token of its own: flat index, tables and order are the same, duplicates rank by slot.
+    return launch_permute(ids, n * topk, 1, n_experts, counts, starts, perm_map, gather_src, active, n_active, scratch,
                           scratch_bytes, nullptr, 0, as_stream(stream));
 }

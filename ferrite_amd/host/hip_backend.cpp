@@ -55,7 +55,7 @@ void DevBuf::download(void* dst, size_t nbytes) const {
 
 struct HipBackend::Api {
 #define FN(name) decltype(&::name) name = nullptr
-    FN(ferrite_kernel_build_id); FN(ferrite_kernel_abi_version); FN(ferrite_hip_last_error);
+    FN(ferrite_kernel_build_id); FN(ferrite_kernel_abi_version); FN(ferrite_hip_last_error); FN(ferrite_hip_warmup);
     FN(ferrite_matmul_f32); FN(ferrite_swiglu_limited_f32); FN(ferrite_moe_route);
     FN(ferrite_rmsnorm_f32); FN(ferrite_hc_post_f32);
     FN(ferrite_moe_packed_bytes); FN(ferrite_moe_pack_weights);
@@ -71,6 +71,7 @@ HipBackend::HipBackend(const std::string& so_path, int device) : api_(new Api) {
     api_->name = reinterpret_cast<decltype(api_->name)>(dlsym(so_, #name));                      \
     if (!api_->name) throw FerriteError(FerriteError::InvalidArg, "missing symbol " #name)
     LOAD(ferrite_kernel_build_id); LOAD(ferrite_kernel_abi_version); LOAD(ferrite_hip_last_error);
+    LOAD(ferrite_hip_warmup);
     LOAD(ferrite_matmul_f32); LOAD(ferrite_swiglu_limited_f32); LOAD(ferrite_moe_route);
     LOAD(ferrite_rmsnorm_f32); LOAD(ferrite_hc_post_f32);
     LOAD(ferrite_moe_packed_bytes); LOAD(ferrite_moe_pack_weights);
@@ -83,6 +84,7 @@ HipBackend::HipBackend(const std::string& so_path, int device) : api_(new Api) {
     hipStream_t s;
     hipck(hipStreamCreate(&s), "hipStreamCreate");   // one stream per backend, default priority
     stream_ = s;
+    ck(api_->ferrite_hip_warmup(), "warmup");   // LDS limits, before anything is captured
 }
 
 HipBackend::~HipBackend() {

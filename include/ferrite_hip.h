@@ -9,7 +9,9 @@
  *     non-zero to FerriteError::InvalidArg); FERRITE_DECLINED means "this shape is outside the kernel's
  *     contract, use another path" (kernels/cuda/dsv41_moe_align.cu:50-52);
  *   - launchers never allocate, never synchronise and never read the environment, so any of them may be
- *     recorded into a stream capture (cuda.rs:3008-3011); all scratch memory comes from the caller;
+ *     recorded into a stream capture (cuda.rs:3008-3011); all scratch memory comes from the caller.  Kernels that
+ *     use more than 64 KiB of LDS need a one-time function attribute per device: ferrite_hip_warmup() sets all of
+ *     them, so that a first call inside a capture makes no runtime call besides its launches;
  *   - matrices are row-major, weights are [out_features, in_features] and ops compute x . w^T
  *     (crates/ferrite-kernel/src/lib.rs:61-66);
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
@@ -30,7 +32,7 @@ extern "C" {
 #define FERRITE_ERR_WORKSPACE 3    /* workspace too small */
 #define FERRITE_ERR_RUNTIME 4      /* a HIP runtime call failed: see ferrite_hip_last_error() */
 
-#define FERRITE_ABI_VERSION 1u
+#define FERRITE_ABI_VERSION 2u
 
 /* dtype tags for activation buffers (ferrite-types DType, crates/ferrite-types/src/lib.rs:16-25) */
 #define FERRITE_DT_F32 0
@@ -48,6 +50,20 @@ unsigned ferrite_kernel_abi_version(void);
 /* Text of the last HIP runtime error seen by this thread ("" if none). */
 const char* ferrite_hip_last_error(void);
 
+/* Once per device, with that device current and outside any stream capture: raises the LDS limit of every kernel
+ * that may need it (the reference warms its pools before a capture for the same reason, cuda.rs:627-657).
+ * Optional for eager use: a launcher that finds its limit too low raises it on the spot. */
+int ferrite_hip_warmup(void);
+
+/* Process-wide test hooks (the reference's counterparts are environment gates read once into a OnceLock,
+ * cuda.rs:5730-5731; here nothing reads the environment).  They change how a layer call tiles its work, and with it
+ * the workspace layout: set them before sizing a workspace, not between sizing and use.
+ *   FERRITE_OVERRIDE_UNIT_ROWS  0 = automatic (default), 16 or 128 = force that token tile for the expert GEMMs
+ *   FERRITE_OVERRIDE_Y_F32      1 = keep the expert outputs `y` in f32 on the 128-row path (default 0: bf16)  */
+#define FERRITE_OVERRIDE_UNIT_ROWS 0
+#define FERRITE_OVERRIDE_Y_F32 1
+int ferrite_hip_set_override(int which, int value);
+
 /* ---- KernelBackend ops on the path (f32 device buffers, like the reference's GLM ABI) ---- */
 
 /* KernelBackend::matmul (lib.rs:73; cpu.rs:82-122): out[n,o] = x[n,k] . w[o,k]^T (+ bias[o], may be NULL).
@@ -62,18 +78,22 @@ int ferrite_swiglu_limited_f32(const float* gate_up, float limit, float* out, in
 /* KernelBackend::moe_route (lib.rs:194-206; cpu.rs:528-572) extended with group-limited selection
  * (n_group = 1 is the reference's router).  probs [n,topk]; ids_f32 [n,topk] (the reference ABI stores ids
  * as f32) and/or ids_i32 [n,topk]; either ids pointer may be NULL.  Requires e <= 512, topk <= 32,
- * e % n_group == 0, topk <= topk_group * e / n_group. */
+ * e % n_group == 0, topk <= topk_group * e / n_group.
+ * NaN scores: CpuBackend panics on them (cpu.rs:560); this op follows the reference's device router instead
+ * (kernels/cuda/ferrite_kernels.cu:1233-1270): a NaN score is never selected, and a slot that no finite score
+ * can fill gets id -1 and weight 0 (it then drops out of the permutation and contributes nothing). */
 int ferrite_moe_route(const float* logits, const float* bias, int n, int e, int topk, int n_group,
                       int topk_group, float routed_scaling, float* probs, float* ids_f32, int32_t* ids_i32,
                       ferrite_stream_t stream);
 
 /* Token permutation by expert (kernels/cuda/dsv41_route.cu:194-315 contract; host golden
  * crates/ferrite-models/src/dsv41/chain_dev.rs:862-899): grouped order = expert ascending, then flat
- * assignment index i = t*topk + j ascending.  ids [n,topk] i32 with distinct experts per token; ids outside
+ * assignment index i = t*topk + j ascending.  ids [n,topk] i32; a token may list an expert more than once (the
+ * reference's vector chain_dev.rs:25042-25061 does): such assignments keep their slot order.  ids outside
  * [0, n_experts) drop out (perm_map = -1).  Outputs: counts[E], starts[E+1], perm_map[n*topk] (original ->
  * grouped), gather_src[n*topk] (grouped -> original, -1 past the end), active[E] (ascending experts with
- * counts > 0, -1 padded), n_active[1].  scratch: ferrite_moe_permute_scratch_bytes(n, n_experts) bytes. */
-size_t ferrite_moe_permute_scratch_bytes(int n, int n_experts);
+ * counts > 0, -1 padded), n_active[1].  scratch: ferrite_moe_permute_scratch_bytes(n, topk, n_experts) bytes. */
+size_t ferrite_moe_permute_scratch_bytes(int n, int topk, int n_experts);
 int ferrite_moe_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* counts, int32_t* starts,
                         int32_t* perm_map, int32_t* gather_src, int32_t* active, int32_t* n_active,
                         void* scratch, size_t scratch_bytes, ferrite_stream_t stream);
@@ -164,14 +184,14 @@ typedef struct ferrite_moe_workspace_view {
     int32_t* n_active;   /* [1] */
     float* y;            /* [(n*topk + n), H] expert outputs in grouped order, then the shared expert's rows; f32,
                           * except bf16 (same shape, half the bytes) when ferrite_moe_layer_unit_rows() is 128 and
-                          * FERRITE_HIP_Y_F32=1 is not set in the environment */
+                          * the FERRITE_OVERRIDE_Y_F32 override is off */
 } ferrite_moe_workspace_view;
 
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
 /* Rows per unit (the token tile of the expert GEMMs) a layer call with these arguments uses: 16 = weights streamed
  * once per unit (decode-sized batches), 128 = both operands tiled through LDS (prefill-sized batches); 0 for an
- * unsupported shape.  The choice is a pure function of (shape, n, mode) and of the environment variable
- * FERRITE_HIP_UNIT_ROWS (16 or 128 forces it, read at every call), like the workspace layout that depends on it.
+ * unsupported shape.  The choice is a pure function of (shape, n, mode) and of the FERRITE_OVERRIDE_UNIT_ROWS
+ * override, like the workspace layout that depends on it.
  * No counterpart in the reference, whose grouped GEMM has one tile shape (dsv41_moe.cu); informational. */
 int ferrite_moe_layer_unit_rows(const ferrite_moe_shape* shape, int n, int mode);
 /* Must run once on a freshly allocated workspace before its first layer call (it clears the arrival counters
@@ -185,7 +205,9 @@ int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int 
 /* The layer.  x [n, H] (x_dtype), out [n, H] (out_dtype).  mode FERRITE_MODE_F32_CHECK reads `w` (checkpoint
  * layout) and requires f32 x; FERRITE_MODE_MFMA_FP8 reads `packed` and w->router_bias.  `packed` carries the
  * router weight, so w->router_w may be NULL with it; the few shapes whose router falls back to the checkpoint
- * layout (n > 65535, very large hidden) then return FERRITE_ERR_INVALID_ARG.
+ * layout (very large hidden) then return FERRITE_ERR_INVALID_ARG.  n > 65535 and routing parameters outside
+ * ferrite_moe_route's limits are refused up front (FERRITE_DECLINED / FERRITE_ERR_INVALID_ARG, as that op returns
+ * them), before anything is enqueued.
  * The launch sequence depends only on (shape, n, mode), never on the routing, so a captured graph of it
  * replays correctly for any input (the GraphCapable contract, crates/ferrite-kernel/src/graph.rs:48-64). */
 int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, const uint8_t* packed,

@@ -76,6 +76,8 @@ def lib() -> C.CDLL:
         L.fo_hc_post.argtypes = [vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int]
         L.fo_moe_route.argtypes = [vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, vp, vp]
         L.fo_moe_route_grouped.argtypes = [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, vp, vp]
+        L.fo_moe_route_grouped_nan.argtypes = [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int,
+                                               vp, vp]
         L.fo_expert_ffn.argtypes = [vp, vp, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int]
         L.fo_moe_permute.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, vp]
         L.fo_moe_align_host.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, vp]
@@ -187,15 +189,18 @@ def hc_post(x, residual, post, comb) -> np.ndarray:
     return out
 
 
-def moe_route(logits, bias, topk: int, routed_scaling: float, n_group: int = 1, topk_group: int = 1):
+def moe_route(logits, bias, topk: int, routed_scaling: float, n_group: int = 1, topk_group: int = 1,
+              nan_policy: int = 0):
+    """nan_policy 0: a NaN score raises (CpuBackend panics); 1: the reference's device router (never selected,
+    unfillable slots get id -1 and weight 0)."""
     lg, b = _f32(logits), _f32(bias)
     n, e = lg.shape
     if b.size != e:
         raise OracleError("router bias shape")
     probs = np.empty((n, topk), np.float32)
     ids = np.empty((n, topk), np.float32)
-    _ck(lib().fo_moe_route_grouped(_p(lg), _p(b), n, e, topk, n_group, topk_group, routed_scaling,
-                                   _p(probs), _p(ids)), "moe_route")
+    _ck(lib().fo_moe_route_grouped_nan(_p(lg), _p(b), n, e, topk, n_group, topk_group, routed_scaling, nan_policy,
+                                       _p(probs), _p(ids)), "moe_route")
     return probs, ids
 
 

@@ -289,40 +289,41 @@ static int scored_cmp(const void* a, const void* b) {
     return (x->j > y->j) - (x->j < y->j);
 }
 
-/* one row of cpu.rs:546-569 given the candidate mask (NULL = all experts) */
+/* one row of cpu.rs:546-569 given the candidate mask (NULL = all experts).
+ * nan_policy 0: a NaN score is an error (partial_cmp().unwrap() panics in the reference);
+ * nan_policy 1: the reference's device router (kernels/cuda/ferrite_kernels.cu:1233-1270): its arg-max
+ *   comparisons are false for NaN, so a NaN score is never selected, and a slot that no finite score can fill
+ *   gets id -1 and weight 0. */
 static int route_row(const float* ls, const float* bs, int e, int topk, float scaling, const uint8_t* keep,
-                     float* sig, scored_t* scored, float* probs, float* ids) {
+                     int nan_policy, float* sig, scored_t* scored, float* probs, float* ids) {
     int nc = 0;
     for (int j = 0; j < e; ++j) {
         sig[j] = 1.0f / (1.0f + expf(-ls[j]));
         float c = sig[j] + bs[j];
-        if (isnan(c)) return 2; /* partial_cmp().unwrap() panics in the reference */
+        if (isnan(c)) {
+            if (nan_policy == 0) return 2;
+            continue;
+        }
         if (!keep || keep[j]) { scored[nc].s = c; scored[nc].j = j; ++nc; }
     }
-    if (topk > nc) return 1;
+    if (topk > nc && nan_policy == 0) return 1;
     qsort(scored, (size_t)nc, sizeof(scored_t), scored_cmp);
+    const int nsel = topk < nc ? topk : nc;
     float sum = 0.0f;
-    for (int r = 0; r < topk; ++r) sum += sig[scored[r].j];
-    for (int r = 0; r < topk; ++r) {
+    for (int r = 0; r < nsel; ++r) sum += sig[scored[r].j];
+    for (int r = 0; r < nsel; ++r) {
         int j = scored[r].j;
         ids[r] = (float)j;
         probs[r] = sig[j] / (sum + FLT_EPSILON) * scaling;
     }
+    for (int r = nsel; r < topk; ++r) { ids[r] = -1.0f; probs[r] = 0.0f; }
     return 0;
 }
 
 /* cpu.rs:528-572 */
 int fo_moe_route(const float* logits, const float* bias, int n, int e, int topk, float routed_scaling,
                  float* probs, float* ids) {
-    if (n < 0 || e <= 0 || topk <= 0 || topk > e) return 1;
-    float* sig = (float*)malloc(sizeof(float) * e);
-    scored_t* sc = (scored_t*)malloc(sizeof(scored_t) * e);
-    int rc = 0;
-    for (int i = 0; i < n && rc == 0; ++i)
-        rc = route_row(logits + (size_t)i * e, bias, e, topk, routed_scaling, NULL, sig, sc,
-                       probs + (size_t)i * topk, ids + (size_t)i * topk);
-    free(sig); free(sc);
-    return rc;
+    return fo_moe_route_grouped_nan(logits, bias, n, e, topk, 1, 1, routed_scaling, 0, probs, ids);
 }
 
 /*
@@ -337,22 +338,35 @@ int fo_moe_route(const float* logits, const float* bias, int n, int e, int topk,
  */
 int fo_moe_route_grouped(const float* logits, const float* bias, int n, int e, int topk, int n_group,
                          int topk_group, float routed_scaling, float* probs, float* ids) {
-    if (n_group <= 1) return fo_moe_route(logits, bias, n, e, topk, routed_scaling, probs, ids);
-    if (n < 0 || e <= 0 || topk <= 0 || e % n_group != 0 || topk_group <= 0 || topk_group > n_group) return 1;
-    int gs = e / n_group;
-    if (topk > topk_group * gs) return 1;
+    return fo_moe_route_grouped_nan(logits, bias, n, e, topk, n_group, topk_group, routed_scaling, 0, probs, ids);
+}
+
+/* The same with the NaN policy of route_row as a parameter.  Under policy 1 a NaN score takes no part in its
+ * group's top-2 either (the comparisons that find them are false for NaN); a group without a finite score
+ * scores -inf (-inf + -inf for two or more experts) and ranks after every group that has one. */
+int fo_moe_route_grouped_nan(const float* logits, const float* bias, int n, int e, int topk, int n_group,
+                             int topk_group, float routed_scaling, int nan_policy, float* probs, float* ids) {
+    if (n < 0 || e <= 0 || topk <= 0 || topk > e) return 1;
+    if (n_group > 1 && (e % n_group != 0 || topk_group <= 0 || topk_group > n_group)) return 1;
+    int gs = n_group > 1 ? e / n_group : e;
+    if (n_group > 1 && topk > topk_group * gs) return 1;
     float* sig = (float*)malloc(sizeof(float) * e);
     scored_t* sc = (scored_t*)malloc(sizeof(scored_t) * e);
-    scored_t* gsc = (scored_t*)malloc(sizeof(scored_t) * n_group);
+    scored_t* gsc = (scored_t*)malloc(sizeof(scored_t) * (n_group > 1 ? n_group : 1));
     uint8_t* keep = (uint8_t*)malloc((size_t)e);
     int rc = 0;
     for (int i = 0; i < n && rc == 0; ++i) {
         const float* ls = logits + (size_t)i * e;
+        if (n_group <= 1) {
+            rc = route_row(ls, bias, e, topk, routed_scaling, NULL, nan_policy, sig, sc, probs + (size_t)i * topk,
+                           ids + (size_t)i * topk);
+            continue;
+        }
         for (int g = 0; g < n_group; ++g) {
             float m1 = -INFINITY, m2 = -INFINITY;
             for (int j = g * gs; j < (g + 1) * gs; ++j) {
                 float c = 1.0f / (1.0f + expf(-ls[j])) + bias[j];
-                if (isnan(c)) rc = 2;
+                if (isnan(c) && nan_policy == 0) rc = 2;
                 if (c > m1) { m2 = m1; m1 = c; }
                 else if (c > m2) m2 = c;
             }
@@ -364,7 +378,7 @@ int fo_moe_route_grouped(const float* logits, const float* bias, int n, int e, i
         memset(keep, 0, (size_t)e);
         for (int r = 0; r < topk_group; ++r)
             for (int j = gsc[r].j * gs; j < (gsc[r].j + 1) * gs; ++j) keep[j] = 1;
-        rc = route_row(ls, bias, e, topk, routed_scaling, keep, sig, sc, probs + (size_t)i * topk,
+        rc = route_row(ls, bias, e, topk, routed_scaling, keep, nan_policy, sig, sc, probs + (size_t)i * topk,
                        ids + (size_t)i * topk);
     }
     free(sig); free(sc); free(gsc); free(keep);

@@ -75,6 +75,11 @@ int fo_moe_route(const float* logits, const float* bias, int n, int e, int topk,
 /* Group-limited variant (no reference counterpart; see header comment). */
 int fo_moe_route_grouped(const float* logits, const float* bias, int n, int e, int topk, int n_group,
                          int topk_group, float routed_scaling, float* probs, float* ids);
+/* The same with the treatment of NaN scores as a parameter: 0 = error 2, as above (CpuBackend panics, cpu.rs:560);
+ * 1 = the reference's device router (kernels/cuda/ferrite_kernels.cu:1233-1270): never selected, unfillable slots
+ * get id -1 and weight 0.  Pinned by its special cases only (no NaN: equal to the above; all NaN: all -1). */
+int fo_moe_route_grouped_nan(const float* logits, const float* bias, int n, int e, int topk, int n_group,
+                             int topk_group, float routed_scaling, int nan_policy, float* probs, float* ids);
 /* cpu.rs:574-625 */
 int fo_expert_ffn(const float* x, const float* gate_w, const float* up_w, const float* down_w, float limit,
                   float* out, int m, int hidden, int inter);

@@ -92,9 +92,19 @@ def test_layer_small_shapes_both_modes(hip, oracle, seed, n):
     assert max_abs_rel(out, oracle.moe_ffn_mxfp4(inp, act_mode=1)["out"]) <= TOL_MFMA
 
 
+@pytest.fixture
+def overrides(hip):
+    """Sets library overrides for one test and puts the defaults back afterwards."""
+    from ferrite_amd.backend import OVERRIDE_UNIT_ROWS, OVERRIDE_Y_F32
+    yield lambda **kw: [hip.set_override({"unit_rows": OVERRIDE_UNIT_ROWS, "y_f32": OVERRIDE_Y_F32}[k], v)
+                        for k, v in kw.items()]
+    hip.set_override(OVERRIDE_UNIT_ROWS, 0)
+    hip.set_override(OVERRIDE_Y_F32, 0)
+
+
 @pytest.mark.parametrize("seed,n,hidden,inter,shared", [(5, 8, 256, 128, 128), (6, 150, 256, 256, 128),
                                                         (7, 700, 384, 256, 384), (8, 1100, 512, 128, 0)])
-def test_unit_rows_128_equals_16(hip, oracle, monkeypatch, seed, n, hidden, inter, shared):
+def test_unit_rows_128_equals_16(hip, oracle, overrides, seed, n, hidden, inter, shared):
     """The 128-row-unit kernels (both operands tiled through LDS) accumulate over k in the same order as the 16-row
     ones: identical bits when both keep the expert outputs in f32, on ragged units (1..128 rows, several units per
     expert, H/64 not a multiple of the block's 4 items).  By default the 128-row path keeps them in bf16: within the
@@ -103,46 +113,18 @@ def test_unit_rows_128_equals_16(hip, oracle, monkeypatch, seed, n, hidden, inte
     inp = synth.make_inputs(cfg, seed=seed)
     layer = hip.load_moe_layer(inp)
     outs = {}
-    monkeypatch.setenv("FERRITE_HIP_Y_F32", "1")
-    for rows in ("16", "128"):
-        monkeypatch.setenv("FERRITE_HIP_UNIT_ROWS", rows)
+    for rows in (16, 128):
+        overrides(unit_rows=rows, y_f32=1)
         layer._ws.clear()
         outs[rows], v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
-    assert np.array_equal(outs["16"], outs["128"])
-    monkeypatch.delenv("FERRITE_HIP_Y_F32")
+    assert np.array_equal(outs[16], outs[128])
+    overrides(y_f32=0)
     layer._ws.clear()
     out_bf16, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
     assert hip.workspace_view(layer, n, MODE_MFMA_FP8)["y"].dtype == torch.bfloat16
     layer._ws.clear()
-    assert max_abs_rel(out_bf16, outs["128"]) <= 2.0 ** -7          # (topk + 1) terms, each within 2^-9 of its f32 value
+    assert max_abs_rel(out_bf16, outs[128]) <= 2.0 ** -7          # (topk + 1) terms, each within 2^-9 of its f32 value
     assert max_abs_rel(out_bf16, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
-
-
-@pytest.mark.parametrize("seed,n,hidden,inter,shared", [(9, 300, 512, 512, 0), (10, 600, 2048, 512, 512),
-                                                        (11, 1100, 1536, 1024, 512)])
-def test_prefill_assembly_loop_equals_16_row_kernels(hip, oracle, monkeypatch, seed, n, hidden, inter, shared):
-    """FERRITE_HIP_PREFILL=asm selects the 128-row kernels whose main loop is one assembly block (weights streamed
-    through registers, activations through a six-stage LDS ring, counted waits).  Same k order as the 16-row
-    kernels: identical bits with f32 expert outputs, for 1, 4 and 3 groups of four k steps in gate/up (the loop's
-    register and stage rotation repeats every 12 steps) and 1 or 2 in down, ragged units, item groups that are not
-    full; bf16 expert outputs within the MFMA bar of the oracle."""
-    cfg = synth.MoeConfig(n, hidden, 8, 3, inter, shared, 4, 2)
-    inp = synth.make_inputs(cfg, seed=seed)
-    layer = hip.load_moe_layer(inp)
-    monkeypatch.setenv("FERRITE_HIP_Y_F32", "1")
-    monkeypatch.setenv("FERRITE_HIP_UNIT_ROWS", "16")
-    layer._ws.clear()
-    ref16, _ = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
-    monkeypatch.setenv("FERRITE_HIP_UNIT_ROWS", "128")
-    monkeypatch.setenv("FERRITE_HIP_PREFILL", "asm")
-    layer._ws.clear()
-    got, _ = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
-    assert np.array_equal(got, ref16)
-    monkeypatch.delenv("FERRITE_HIP_Y_F32")
-    layer._ws.clear()
-    got_bf16, _ = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
-    layer._ws.clear()
-    assert max_abs_rel(got_bf16, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA
 
 
 def test_layer_c1_decode(hip, oracle):

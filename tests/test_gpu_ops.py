@@ -121,6 +121,53 @@ def test_moe_route_extreme_logits(hip, oracle):
     assert np.array_equal(i, io) and np.array_equal(p, po)
 
 
+def test_moe_route_nan_scores(hip, oracle):
+    """NaN logits: never selected; slots that no finite score can fill get id -1 and weight 0, as the reference's
+    device router leaves them (kernels/cuda/ferrite_kernels.cu:1233-1270).  Bit-equal to the oracle's statement of
+    that policy, grouped and ungrouped, and through the fused layer: such slots contribute nothing."""
+    rng = np.random.default_rng(11)
+    logits = rng.normal(0, 1.5, (8, 64)).astype(np.float32)
+    bias = rng.normal(0, 0.01, 64).astype(np.float32)
+    logits[0, 5] = np.nan
+    logits[1, :] = np.nan
+    logits[2, :61] = np.nan
+    logits[3, 16:32] = np.nan
+    logits[4, ::2] = np.nan
+    for ng, tg in ((1, 1), (4, 2)):
+        p, i = route(hip, logits, bias, 6, 2.5, ng, tg)
+        po, io = oracle.moe_route(logits, bias, 6, 2.5, ng, tg, nan_policy=1)
+        assert np.array_equal(i, io), (ng, tg)
+        assert np.array_equal(p, po), (ng, tg)
+    assert i[1].tolist() == [-1] * 6 and p[1].tolist() == [0.0] * 6
+
+
+def test_layer_with_nan_activations_keeps_other_tokens_intact(hip, oracle):
+    """A token whose activations are NaN routes nowhere (ids -1, no row in the permutation); every other token's row
+    is bit-identical to a run without it, in both the fused-head and the separate-launch path."""
+    from ferrite_amd import synth
+    from ferrite_amd.backend import MODE_MFMA_FP8
+    for n in (24, 300):
+        cfg = synth.MoeConfig(n, 256, 16, 4, 128, 128, 4, 2)
+        inp = synth.make_inputs(cfg, seed=n)
+        layer = hip.load_moe_layer(inp)
+        x = torch.from_numpy(inp.x).to(hip.device)
+        out = torch.empty_like(x)
+        hip.moe_layer_dev_mxfp4(layer, x, out, MODE_MFMA_FP8)
+        hip.sync()
+        clean = out.cpu().numpy()
+        x[7, :] = float("nan")
+        hip.moe_layer_dev_mxfp4(layer, x, out, MODE_MFMA_FP8)
+        hip.sync()
+        got = out.cpu().numpy()
+        v = hip.workspace_view(layer, n, MODE_MFMA_FP8)
+        assert v["ids"][7].cpu().tolist() == [-1] * 4
+        assert v["perm_map"].view(n, 4)[7].cpu().tolist() == [-1] * 4
+        keep = np.arange(n) != 7
+        assert np.array_equal(got[keep], clean[keep])
+        # (row 7 itself holds whatever the shared expert makes of the quantised row: the reference's e4m3 encoder
+        # saturates non-finite values to +-448, quant.rs:98-124, so it need not be NaN)
+
+
 def test_moe_route_shape_errors(hip):
     z = lambda *s: torch.zeros(*s, device=hip.device)
     with pytest.raises(InvalidArg):
@@ -138,13 +185,32 @@ def permute(hip, ids, e):
     return {k: v.cpu().numpy() for k, v in t.items()}
 
 
-def test_moe_permute_reference_vector(hip):  # chain_dev.rs:25042-25061 routing table
-    t = permute(hip, np.array([[5, 1, 5], [1, 5, 2], [9, 1, 9]]), 12)
-    # NB the reference table repeats an expert inside a token (5,1,5 / 9,1,9); the device contract needs distinct
-    # experts per token, so only the tokens' first occurrences are meaningful here: use the distinct variant below
+def test_moe_permute_reference_vector(hip, oracle):  # chain_dev.rs:25042-25061 routing table, as it stands there
+    """The reference's vector lists an expert twice inside a token (5,1,5 and 9,1,9); its order is
+    [1,3,7] [5] [0,2,4] [6,8] for experts 1, 2, 5, 9 with counts 3, 1, 3, 2."""
+    ids = np.array([[5, 1, 5], [1, 5, 2], [9, 1, 9]])
+    t = permute(hip, ids, 12)
+    assert t["gather_src"].tolist() == [1, 3, 7, 5, 0, 2, 4, 6, 8]
+    assert t["counts"].tolist() == [0, 3, 1, 0, 0, 3, 0, 0, 0, 2, 0, 0]
+    assert t["active"][:4].tolist() == [1, 2, 5, 9] and int(t["n_active"][0]) == 4
+    o = oracle.moe_permute(ids, 12)
+    for key in ("counts", "starts", "perm_map", "gather_src", "active"):
+        assert np.array_equal(t[key], o[key]), key
     t = permute(hip, np.array([[5, 1, 7], [1, 5, 2], [9, 1, 3]]), 12)
     assert t["gather_src"].tolist() == [1, 3, 7, 5, 8, 0, 4, 2, 6]
     assert t["counts"].tolist() == [0, 3, 1, 1, 0, 2, 0, 1, 0, 1, 0, 0]
+
+
+@pytest.mark.parametrize("n,k,e", [(40, 6, 5), (700, 8, 16), (3000, 4, 3)])
+def test_moe_permute_repeated_experts_in_a_token(hip, oracle, n, k, e):
+    """ids drawn with replacement: many tokens repeat an expert; also beyond the single-block path."""
+    rng = np.random.default_rng(n)
+    ids = rng.integers(0, e, (n, k)).astype(np.int32)
+    t = permute(hip, ids, e)
+    o = oracle.moe_permute(ids, e)
+    for key in ("counts", "starts", "perm_map", "gather_src", "active"):
+        assert np.array_equal(t[key], o[key]), key
+    assert np.array_equal(t["gather_src"], np.argsort(ids.ravel(), kind="stable"))
 
 
 @pytest.mark.parametrize("n,k,e", [(1, 1, 1), (7, 3, 5), (32, 8, 128), (192, 8, 128), (1000, 8, 256), (1024, 8, 128),

@@ -37,12 +37,58 @@ def test_bench_refuses_more_than_one_gpu():
         assert "one GPU" in res.stderr and res.stdout == ""
 
 
-def test_generated_assembly_loop_is_current(tmp_path):
-    """csrc/prefill_mainloop_asm.inc is what csrc/gen_prefill_asm.py writes."""
+def _layer_rc(lib, backend, n, **over):
+    """Return code of the layer call for a shape; argument checks run before any pointer is used or any GPU call is
+    made, so dummy non-null pointers do on a machine without a GPU."""
+    base = dict(hidden=256, n_experts=64, topk=4, inter=128, shared_inter=128, n_group=4, topk_group=2,
+                routed_scaling=2.5, swiglu_limit=10.0)
+    base.update(over)
+    shape = backend.MoeShape(*[base[k] for k, _ in backend.MoeShape._fields_])
+    w = backend.MoeWeights()
+    dummy = C.c_void_p(4096)
+    return lib.ferrite_moe_layer_mxfp4(C.byref(shape), C.byref(w), dummy, dummy, backend.DT_F32, n, dummy,
+                                       backend.DT_F32, backend.MODE_MFMA_FP8, dummy, 1 << 30, None)
+
+
+def test_layer_refuses_routing_parameters_outside_the_kernels_limits():
+    """The fused head (decode-sized batches) and the separate routing launches refuse the same parameters, up front:
+    what ferrite_moe_route returns for them, at 32 tokens as at 4096."""
+    from ferrite_amd import backend
+    lib = backend.load_library()
+    for n in (32, 4096):
+        assert _layer_rc(lib, backend, n, n_experts=64, topk=33, n_group=1, topk_group=1) == backend.DECLINED
+        assert _layer_rc(lib, backend, n, n_experts=130, topk=4, n_group=65, topk_group=33) == backend.DECLINED
+        assert _layer_rc(lib, backend, n, n_experts=66, topk=4, n_group=4, topk_group=2) == backend.ERR_INVALID_ARG
+        assert _layer_rc(lib, backend, n, n_experts=64, topk=4, n_group=4, topk_group=0) == backend.ERR_INVALID_ARG
+        assert _layer_rc(lib, backend, n, n_experts=64, topk=40, n_group=4, topk_group=2) == backend.ERR_INVALID_ARG
+        assert _layer_rc(lib, backend, n, n_experts=1024, topk=4, n_group=1, topk_group=1) == backend.DECLINED
+    # more tokens than a launch's grid.y takes: refused before anything is enqueued, not half way through
+    assert _layer_rc(lib, backend, 65536) == backend.DECLINED
+    assert _layer_rc(lib, backend, 0) == backend.ERR_INVALID_ARG
+
+
+def test_overrides_validate_their_arguments():
+    from ferrite_amd import backend
+    lib = backend.load_library()
+    assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 64) == backend.ERR_INVALID_ARG
+    assert lib.ferrite_hip_set_override(backend.OVERRIDE_Y_F32, 2) == backend.ERR_INVALID_ARG
+    assert lib.ferrite_hip_set_override(7, 0) == backend.ERR_INVALID_ARG
+    shape = backend.MoeShape(4096, 128, 8, 1536, 1536, 8, 4, 2.5, 10.0)
+    assert lib.ferrite_moe_layer_unit_rows(C.byref(shape), 32, backend.MODE_MFMA_FP8) == 16
+    assert lib.ferrite_moe_layer_unit_rows(C.byref(shape), 4096, backend.MODE_MFMA_FP8) == 128
+    assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 128) == backend.OK
+    assert lib.ferrite_moe_layer_unit_rows(C.byref(shape), 32, backend.MODE_MFMA_FP8) == 128
+    assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 0) == backend.OK
+    assert lib.ferrite_moe_layer_unit_rows(C.byref(shape), 32, backend.MODE_MFMA_FP8) == 16
+
+
+def test_library_sources_read_no_environment():
+    """Launchers may be recorded into a stream capture; the reference reads its gates once for that reason
+    (cuda.rs:5730-5731).  Here no source of the library reads the environment at all."""
     csrc = os.path.join(ROOT, "ferrite_amd", "csrc")
-    out = str(tmp_path / "loop.inc")
-    subprocess.run([os.sys.executable, os.path.join(csrc, "gen_prefill_asm.py"), out], check=True, capture_output=True)
-    assert open(out).read() == open(os.path.join(csrc, "prefill_mainloop_asm.inc")).read()
+    for name in sorted(os.listdir(csrc)):
+        text = open(os.path.join(csrc, name)).read()
+        assert "getenv" not in text, name
 
 
 def test_backend_refuses_to_run_without_gpu_or_library(tmp_path):

@@ -310,3 +310,40 @@ def test_hc_post_reference_fixture_and_special_cases(oracle):
     assert np.array_equal(oracle.hc_post(x, res, post, np.zeros_like(comb)), post[:, :, None] * x[:, None, :])
     with pytest.raises(oracle.OracleError):
         oracle.hc_post(x, res, post[:, :2], comb)
+
+
+def test_route_nan_scores_device_policy(oracle):
+    """CpuBackend panics on a NaN score (cpu.rs:560: partial_cmp().unwrap()); the reference's device router never
+    selects one and marks slots it cannot fill with id -1, weight 0 (kernels/cuda/ferrite_kernels.cu:1233-1270).
+    The oracle states both; the second is pinned by its special cases: without NaN it is the first, a NaN expert
+    is as good as absent (the remaining experts route as if it scored -inf), all-NaN gives all -1."""
+    rng = np.random.default_rng(5)
+    logits = rng.normal(0, 1.5, (6, 32)).astype(np.float32)
+    bias = rng.normal(0, 0.01, 32).astype(np.float32)
+    for ng, tg in ((1, 1), (4, 2)):
+        p0, i0 = oracle.moe_route(logits, bias, 4, 2.5, ng, tg)
+        p1, i1 = oracle.moe_route(logits, bias, 4, 2.5, ng, tg, nan_policy=1)
+        assert np.array_equal(p0, p1) and np.array_equal(i0, i1)
+    bad = logits.copy()
+    bad[0, 3] = np.nan
+    bad[1, :] = np.nan
+    bad[2, :30] = np.nan          # two finite scores for four slots
+    with pytest.raises(oracle.OracleError):
+        oracle.moe_route(bad, bias, 4, 2.5)
+    p, i = oracle.moe_route(bad, bias, 4, 2.5, nan_policy=1)
+    # row 0: expert 3 absent == the same row with a hugely negative logit there (sigmoid 0, bias cannot lift it)
+    sub = logits[:1].copy()
+    sub[0, 3] = -1e30
+    big_neg_bias = bias.copy()
+    big_neg_bias[3] = -10.0
+    ps, is_ = oracle.moe_route(sub, big_neg_bias, 4, 2.5)
+    assert np.array_equal(i[0], is_[0]) and np.array_equal(p[0], ps[0]) and 3 not in i[0]
+    assert i[1].tolist() == [-1, -1, -1, -1] and p[1].tolist() == [0, 0, 0, 0]
+    assert sorted(i[2, :2].tolist()) == [30, 31] and i[2, 2:].tolist() == [-1, -1] and p[2, 2:].tolist() == [0, 0]
+    assert abs(p[2, :2].sum() - 2.5) < 1e-5
+    assert np.array_equal(i[3:], oracle.moe_route(logits, bias, 4, 2.5)[1][3:])
+    # grouped: a group whose experts are all NaN ranks last and is dropped when enough other groups exist
+    g = logits.copy()
+    g[:, 8:16] = np.nan
+    pg, ig = oracle.moe_route(g, bias, 4, 2.5, 4, 2, nan_policy=1)
+    assert ((ig < 8) | (ig >= 16)).all() and (ig >= 0).all()
