@@ -63,6 +63,7 @@ class MoeWeights(C.Structure):
 
 
 STAGE_EVENTS = 10   # FERRITE_MOE_STAGE_EVENTS
+STATIC_WORKSPACE_BYTES = 16 << 20   # FERRITE_STATIC_WORKSPACE_BYTES
 
 
 class MoeExpertSrc(C.Structure):
@@ -87,7 +88,7 @@ EXPORTS = [
     "ferrite_mxfp4_dequant", "ferrite_mxfp4_quant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes",
     "ferrite_moe_pack_weights", "ferrite_moe_pack_expert", "ferrite_moe_pack_router",
     "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_block_workspace_bytes", "ferrite_moe_block_mxfp4", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
-    "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_timed", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
+    "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_static", "ferrite_moe_layer_mxfp4_timed", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
     "ferrite_graph_destroy",
 ]
 
@@ -133,6 +134,8 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_moe_layer_mxfp4.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp, i32, i32, vp, i32,
                                             i32, vp, sz, vp]
     lib.ferrite_moe_layer_mxfp4_timed.argtypes = lib.ferrite_moe_layer_mxfp4.argtypes + [C.POINTER(vp)]
+    lib.ferrite_moe_layer_mxfp4_static.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp, i32, i32, vp, i32,
+                                                   i32, vp]
     lib.ferrite_graph_begin.argtypes = [vp]
     lib.ferrite_graph_end.argtypes = [vp, C.POINTER(vp)]
     lib.ferrite_graph_launch.argtypes = [vp, vp]
@@ -545,6 +548,27 @@ class HipBackend:
             if len(stage_events) != STAGE_EVENTS:
                 raise InvalidArg(f"stage_events must hold {STAGE_EVENTS} event handles")
             self._ck(self.lib.ferrite_moe_layer_mxfp4_timed(*args, stage_events), "moe_layer_mxfp4")
+
+    def moe_layer_dev_mxfp4_static(self, layer: MoeLayer, x: torch.Tensor, out: torch.Tensor, mode: int = MODE_MFMA_FP8):
+        """The same layer on the library's built-in workspace: nothing is allocated, here or in the library."""
+        self.recorder.record("moe_layer_mxfp4")
+        self._leave()
+        cfg = layer.cfg
+        if x.dim() != 2 or x.shape[1] != cfg.hidden:
+            raise ShapeMismatch(f"x {tuple(x.shape)} vs hidden {cfg.hidden}")
+        n = x.shape[0]
+        if tuple(out.shape) != (n, cfg.hidden):
+            raise InvalidArg(f"out shape {tuple(out.shape)} != [{n},{cfg.hidden}]")
+        dts = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
+        if x.dtype not in dts or out.dtype not in dts or not x.is_contiguous() or not out.is_contiguous():
+            raise InvalidArg("x/out must be contiguous f32 or bf16 device tensors")
+        self._enter()
+        rc = self.lib.ferrite_moe_layer_mxfp4_static(
+            C.byref(layer.shape), C.byref(layer.weights), None if layer.packed is None else layer.packed.data_ptr(),
+            x.data_ptr(), dts[x.dtype], n, out.data_ptr(), dts[out.dtype], mode, self._st())
+        if rc == ERR_WORKSPACE:
+            raise FerriteError(self.lib.ferrite_hip_last_error().decode())
+        self._ck(rc, "moe_layer_mxfp4_static")
 
     def block_workspace(self, layer: MoeLayer, n: int, mode: int) -> torch.Tensor:
         key = ("block", n, mode)

@@ -153,10 +153,14 @@ extern "C" int ferrite_hip_set_override(int which, int value) {
     return FERRITE_ERR_INVALID_ARG;
 }
 
+static int static_workspace(void** out);
+
 extern "C" int ferrite_hip_warmup(void) {
     int rc;
     if ((rc = warmup_route())) return rc;
-    return warmup_experts_mfma();
+    if ((rc = warmup_experts_mfma())) return rc;
+    void* ws = nullptr;
+    return static_workspace(&ws);   // resolves this device's copy of the built-in workspace
 }
 
 extern "C" int ferrite_moe_layer_unit_rows(const ferrite_moe_shape* shape, int n, int mode) {
@@ -341,6 +345,51 @@ extern "C" int ferrite_moe_layer_mxfp4_timed(const ferrite_moe_shape* shape, con
                                              ferrite_stream_t stream, void* const* stage_events) {
     return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, workspace, workspace_bytes, stream,
                           stage_events);
+}
+
+// ---- the layer for callers that cannot allocate: its workspace is a file-scope device array ----
+// Each GPU the library runs on holds its own copy of the array, at its own address, until the process ends.  The
+// array's name is a host-side stand-in for it, not a device address: host code uses the address that
+// hipGetSymbolAddress returns for the current device, kept per device.
+static __device__ __align__(256) unsigned char scratch[FERRITE_STATIC_WORKSPACE_BYTES];
+
+static int static_workspace(void** out) {
+    static std::mutex mu;
+    static void* ptrs[kMaxDevices] = {};
+    int dev = 0;
+    if (int rc = current_device(&dev)) return rc;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress");
+        if (!p || (reinterpret_cast<uintptr_t>(p) & 255)) return FERRITE_ERR_RUNTIME;
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return FERRITE_OK;
+}
+
+extern "C" int ferrite_moe_layer_mxfp4_static(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
+                                              const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
+                                              int out_dtype, int mode, ferrite_stream_t stream) {
+    int rc = check_shape(shape, n, mode);
+    if (rc) return rc;
+    const Workspace w = carve(*shape, n, mode);
+    if (w.total > FERRITE_STATIC_WORKSPACE_BYTES) {
+        snprintf(g_last_error, sizeof(g_last_error),
+                 "ferrite_moe_layer_mxfp4_static: this call needs %zu bytes of workspace, the built-in one holds %zu",
+                 w.total, (size_t)FERRITE_STATIC_WORKSPACE_BYTES);
+        return FERRITE_ERR_WORKSPACE;
+    }
+    void* ws = nullptr;
+    if ((rc = static_workspace(&ws))) return rc;
+    // The array keeps what the last call left in it.  Only the arrival counters have to start at zero; a call that
+    // ran to its end leaves them so, one that was cut short may not have: cleared here, by a kernel (capturable).
+    if ((rc = launch_zero_i32(reinterpret_cast<int32_t*>(static_cast<char*>(ws) + w.counters), n + 1, as_stream(stream))))
+        return rc;
+    return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, ws, FERRITE_STATIC_WORKSPACE_BYTES,
+                          stream, nullptr);
 }
 
 // ---- rmsnorm -> layer -> hc_post (exec/lib.rs:487-492) ----

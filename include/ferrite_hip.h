@@ -214,6 +214,22 @@ int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_we
                             const void* x, int x_dtype, int n, void* out, int out_dtype, int mode,
                             void* workspace, size_t workspace_bytes, ferrite_stream_t stream);
 
+/* The same layer for callers that cannot allocate device memory at all and so have no workspace to pass: code
+ * under a stream capture that arrives without buffers, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference, whose callers always own a DevBuf pool (cuda.rs:558-744).  The workspace is an
+ * array of FERRITE_STATIC_WORKSPACE_BYTES built into the library (each GPU the library runs on holds one copy until
+ * the process ends); inputs, weights and outputs are still the caller's.  Same results as ferrite_moe_layer_mxfp4,
+ * bit for bit.  Calls whose workspace (ferrite_moe_layer_workspace_bytes) exceeds the array return
+ * FERRITE_ERR_WORKSPACE with the two sizes in ferrite_hip_last_error(); at H 4096, top-8, I 1536 that is up to
+ * about 100 tokens.  It calls no hipMalloc / hipFree or anything else that allocates, and does not synchronise; the
+ * first call on a device looks the array's address up (ferrite_hip_warmup() does that ahead of time, e.g. before a
+ * capture).  Every call on a GPU uses that GPU's one array: calls that overlap on the same GPU (two streams, two
+ * threads) race, and the workspace-view entry points do not apply. */
+#define FERRITE_STATIC_WORKSPACE_BYTES (16u << 20)
+int ferrite_moe_layer_mxfp4_static(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, const uint8_t* packed,
+                                   const void* x, int x_dtype, int n, void* out, int out_dtype, int mode,
+                                   ferrite_stream_t stream);
+
 /* ---- the steps on either side of the layer (crates/ferrite-exec/src/lib.rs:487-492) ---- */
 
 /* KernelBackend::rmsnorm (crates/ferrite-kernel/src/lib.rs:76; CpuBackend, cpu.rs:124-143; CUDA: ferrite_rmsnorm,

@@ -67,6 +67,25 @@ def test_layer_refuses_routing_parameters_outside_the_kernels_limits():
     assert _layer_rc(lib, backend, 0) == backend.ERR_INVALID_ARG
 
 
+def test_static_workspace_entry_refuses_oversize_before_touching_a_gpu():
+    """The size check of ferrite_moe_layer_mxfp4_static is host arithmetic: it answers without a GPU."""
+    from ferrite_amd import backend
+    lib = backend.load_library()
+    shape = backend.MoeShape(4096, 128, 8, 1536, 1536, 8, 4, 2.5, 10.0)
+    w = backend.MoeWeights()
+    d = C.c_void_p(4096)
+    need = lib.ferrite_moe_layer_workspace_bytes(C.byref(shape), 192, backend.MODE_MFMA_FP8)
+    assert need > backend.STATIC_WORKSPACE_BYTES
+    rc = lib.ferrite_moe_layer_mxfp4_static(C.byref(shape), C.byref(w), d, d, backend.DT_BF16, 192, d, backend.DT_BF16,
+                                            backend.MODE_MFMA_FP8, None)
+    assert rc == backend.ERR_WORKSPACE
+    msg = lib.ferrite_hip_last_error().decode()
+    assert str(need) in msg and str(backend.STATIC_WORKSPACE_BYTES) in msg
+    assert lib.ferrite_moe_layer_workspace_bytes(C.byref(shape), 32, backend.MODE_MFMA_FP8) <= backend.STATIC_WORKSPACE_BYTES
+    hdr = open(os.path.join(ROOT, "include", "ferrite_hip.h")).read()
+    assert "#define FERRITE_STATIC_WORKSPACE_BYTES (16u << 20)" in hdr and backend.STATIC_WORKSPACE_BYTES == 16 << 20
+
+
 def test_overrides_validate_their_arguments():
     from ferrite_amd import backend
     lib = backend.load_library()
