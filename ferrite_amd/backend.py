@@ -28,7 +28,7 @@ ABI_VERSION = 2
 
 OK, ERR_INVALID_ARG, DECLINED, ERR_WORKSPACE, ERR_RUNTIME = 0, 1, 2, 3, 4
 DT_F32, DT_BF16 = 0, 1
-MODE_F32_CHECK, MODE_MFMA_FP8 = 0, 1
+MODE_F32_CHECK, MODE_MFMA_FP8, MODE_MFMA_FP8_X2 = 0, 1, 2
 OVERRIDE_UNIT_ROWS, OVERRIDE_Y_F32 = 0, 1
 
 
@@ -85,7 +85,8 @@ EXPORTS = [
     "ferrite_kernel_build_id", "ferrite_kernel_abi_version", "ferrite_hip_last_error", "ferrite_hip_warmup",
     "ferrite_hip_set_override", "ferrite_matmul_f32", "ferrite_rmsnorm_f32", "ferrite_hc_post_f32",
     "ferrite_swiglu_limited_f32", "ferrite_moe_route", "ferrite_moe_permute_scratch_bytes", "ferrite_moe_permute",
-    "ferrite_mxfp4_dequant", "ferrite_mxfp4_quant", "ferrite_act_quant_fp8", "ferrite_moe_packed_bytes",
+    "ferrite_mxfp4_dequant", "ferrite_mxfp4_quant", "ferrite_act_quant_fp8", "ferrite_act_quant_fp8_x2",
+    "ferrite_moe_packed_bytes",
     "ferrite_moe_pack_weights", "ferrite_moe_pack_expert", "ferrite_moe_pack_router",
     "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_block_workspace_bytes", "ferrite_moe_block_mxfp4", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
     "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_static", "ferrite_moe_layer_mxfp4_timed", "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
@@ -115,6 +116,7 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_moe_permute.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     lib.ferrite_mxfp4_dequant.argtypes = [vp, vp, i64, i64, vp, vp]
     lib.ferrite_act_quant_fp8.argtypes = [vp, i32, i64, i32, vp, vp, vp]
+    lib.ferrite_act_quant_fp8_x2.argtypes = [vp, i32, i64, i32, vp, vp, vp, vp, vp]
     lib.ferrite_mxfp4_quant.argtypes = [vp, i32, i64, i64, vp, vp, vp]
     lib.ferrite_moe_pack_expert.argtypes = [vp, i32, vp, vp, vp]
     lib.ferrite_moe_pack_router.argtypes = [vp, vp, vp, vp]
@@ -469,6 +471,22 @@ class HipBackend:
         self._leave()
         return q, s
 
+    def act_quant_fp8_x2(self, x: torch.Tensor):
+        """Two-term e4m3-per-32 quantisation: (q1, s1, q2, s2), the second pair from the residual of the first."""
+        if x.dtype not in (torch.float32, torch.bfloat16) or x.dim() != 2 or not x.is_contiguous():
+            raise InvalidArg("x must be contiguous [rows, cols] f32 or bf16")
+        rows, cols = x.shape
+        if cols % 32:
+            raise InvalidArg("cols must be a multiple of 32")
+        mk = lambda c: torch.empty((rows, c), dtype=torch.uint8, device=self.device)
+        q1, s1, q2, s2 = mk(cols), mk(cols // 32), mk(cols), mk(cols // 32)
+        self._enter()
+        self._ck(self.lib.ferrite_act_quant_fp8_x2(x.data_ptr(), DT_F32 if x.dtype == torch.float32 else DT_BF16, rows,
+                                                   cols, q1.data_ptr(), s1.data_ptr(), q2.data_ptr(), s2.data_ptr(),
+                                                   self._st()), "act_quant_fp8_x2")
+        self._leave()
+        return q1, s1, q2, s2
+
     # ---- the fused layer ----
     def load_moe_layer(self, inp: MoeInputs, keep_checkpoint_layout: bool = True, pack: bool = True) -> MoeLayer:
         """Upload one layer's weights (checkpoint layout) and build the packed tile layout on the device."""
@@ -535,7 +553,7 @@ class HipBackend:
         dts = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
         if x.dtype not in dts or out.dtype not in dts or not x.is_contiguous() or not out.is_contiguous():
             raise InvalidArg("x/out must be contiguous f32 or bf16 device tensors")
-        if mode == MODE_MFMA_FP8 and layer.packed is None:
+        if mode != MODE_F32_CHECK and layer.packed is None:
             raise InvalidArg("layer has no packed weights")
         ws = workspace if workspace is not None else self.workspace(layer, n, mode)
         self._enter()
@@ -602,7 +620,7 @@ class HipBackend:
         for t, nm in ((li, "li"), (norm_w, "norm_w"), (residual, "residual"), (post, "post"), (comb, "comb"),
                       (out, "out")):
             self._dev(t, torch.float32, nm)
-        if mode == MODE_MFMA_FP8 and layer.packed is None:
+        if mode != MODE_F32_CHECK and layer.packed is None:
             raise InvalidArg("layer has no packed weights")
         ws = self.block_workspace(layer, n, mode)
         blk = MoeBlockArgs(norm_w.data_ptr(), eps, residual.data_ptr(), post.data_ptr(), comb.data_ptr(), nh)

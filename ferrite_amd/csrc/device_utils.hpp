@@ -42,11 +42,9 @@ __device__ __forceinline__ float swiglu_fast(float g, float u, float limit) {
     return gi * __builtin_amdgcn_rcpf(1.0f + __expf(-gi)) * ui;
 }
 
-// act_quant_fp8 of one block of 32 consecutive values (crates/ferrite-models/src/dsv41/quant.rs:190-214,
-// power-of-two scale): 32 e4m3 codes to q (32-byte aligned) and the e8m0 scale byte as the return value.
+// 32 consecutive f32 / bf16 values (32- / 16-byte aligned) into registers.
 template <typename XT>
-__device__ __forceinline__ uint32_t quant_block32(const XT* __restrict__ src, uint8_t* __restrict__ q) {
-    float v[32];
+__device__ __forceinline__ void load_block32(const XT* __restrict__ src, float (&v)[32]) {
     if constexpr (sizeof(XT) == 4) {
         const float4* p = reinterpret_cast<const float4*>(src);
 #pragma unroll
@@ -67,20 +65,54 @@ __device__ __forceinline__ uint32_t quant_block32(const XT* __restrict__ src, ui
             }
         }
     }
+}
+
+// act_quant_fp8 of one block of 32 values held in registers (crates/ferrite-models/src/dsv41/quant.rs:190-214,
+// power-of-two scale): 32 e4m3 codes to q (32-byte aligned) and the e8m0 scale byte as the return value.
+// kResidual: v is replaced by what the codes leave over, v - decode(code) * scale (one f32 multiply by a power of
+// two and one f32 subtraction per value), the input of the second term of a two-term quantisation.
+template <bool kResidual>
+__device__ __forceinline__ uint32_t encode_block32(float (&v)[32], uint8_t* __restrict__ q) {
     float amax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
     const uint32_t sb = block_scale_e8m0(amax);
     const float inv = u2f((254u - sb) << 23);   // 2^(127 - sb): exact reciprocal of the power-of-two scale
+    const float sc = u2f(sb << 23);
     uint32_t out[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         out[i] = e4m3_encode4_hw(v[4 * i] * inv, v[4 * i + 1] * inv, v[4 * i + 2] * inv, v[4 * i + 3] * inv);
+        if constexpr (kResidual) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                v[4 * i + j] = fadd(v[4 * i + j], -fmul(e4m3_decode((out[i] >> (8 * j)) & 0xffu), sc));
+        }
     }
     uint4* o = reinterpret_cast<uint4*>(q);
     o[0] = make_uint4(out[0], out[1], out[2], out[3]);
     o[1] = make_uint4(out[4], out[5], out[6], out[7]);
     return sb;
+}
+
+// act_quant_fp8 of one block of 32 consecutive values in memory.
+template <typename XT>
+__device__ __forceinline__ uint32_t quant_block32(const XT* __restrict__ src, uint8_t* __restrict__ q) {
+    float v[32];
+    load_block32(src, v);
+    return encode_block32<false>(v, q);
+}
+
+// Two-term quantisation of one block: x ~ decode(q1) * 2^(s1-127) + decode(q2) * 2^(s2-127), where the second
+// term is act_quant_fp8 of the residual of the first.  Returns s1 | s2 << 8.
+template <typename XT>
+__device__ __forceinline__ uint32_t quant_block32_x2(const XT* __restrict__ src, uint8_t* __restrict__ q1,
+                                                     uint8_t* __restrict__ q2) {
+    float v[32];
+    load_block32(src, v);
+    const uint32_t s1 = encode_block32<true>(v, q1);
+    const uint32_t s2 = encode_block32<false>(v, q2);
+    return s1 | (s2 << 8);
 }
 
 }  // namespace fe

@@ -175,17 +175,28 @@ __device__ __forceinline__ void stream_item(StreamRegs& r, const u4v* __restrict
 }
 
 // Copies the e4m3 rows of a unit into LDS in B-operand order and builds the packed scale words.
-// row_src(c) gives the source row index of column c (or -1).  q rows are K bytes; scale rows are in operand
-// order (scale_pos), scale_pitch(K) bytes long.
-template <typename RowFn>
-__device__ __forceinline__ void fill_b_operand(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs, int K,
-                                               int nrows, RowFn row_src, u4v* bq, uint32_t* bsc) {
+// row_src(r) gives the source row of unit row r (or -1).  Source rows are `pitch` bytes apart, of which the first K
+// are read; scale rows are in operand order (scale_pos), `spitch` bytes apart.
+// kX2: the activations are two-term (value ~ term 1 + term 2, each e4m3 per 32 with its own scales, in two planes
+// of the same shape).  A unit then has at most 8 rows, and the 16 operand columns hold term 1 of row c in column c
+// and term 2 of row c in column c + 8: one instruction multiplies both terms by the weights, and the two partial
+// results of a row meet in the epilogue (lanes c and c ^ 8).  No more instructions and no more LDS than one term
+// for 16 rows.
+template <bool kX2, typename RowFn>
+__device__ __forceinline__ void fill_b_operand(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs,
+                                               const uint8_t* __restrict__ q2, const uint8_t* __restrict__ qs2, int K,
+                                               size_t pitch, int spitch, int nrows, RowFn row_src, u4v* bq,
+                                               uint32_t* bsc) {
     const int chunks = K / 16;
-    for (int idx = threadIdx.x; idx < nrows * chunks; idx += blockDim.x) {
+    const int ncols = kX2 ? 16 : nrows;
+    for (int idx = threadIdx.x; idx < ncols * chunks; idx += blockDim.x) {
         const int c = idx / chunks, j = idx % chunks;
-        const int r = row_src(c);
+        const int ur = kX2 ? (c & 7) : c;
+        if (kX2 && ur >= nrows) continue;
+        const int r = row_src(ur);
+        const uint8_t* plane = (kX2 && c >= 8) ? q2 : q;
         u4v v = {0u, 0u, 0u, 0u};
-        if (r >= 0) v = *reinterpret_cast<const u4v*>(q + (size_t)r * K + (size_t)j * 16);
+        if (r >= 0) v = *reinterpret_cast<const u4v*>(plane + (size_t)r * pitch + (size_t)j * 16);
         const int k = j * 16, kt = k >> 7, within = k & 127;
         const int half = within >> 6, g = (within & 63) >> 4;
         bq[(kt * 2 + half) * 64 + g * 16 + c] = v;
@@ -193,13 +204,23 @@ __device__ __forceinline__ void fill_b_operand(const uint8_t* __restrict__ q, co
     const int KT = K / 128, KT4 = (KT + 3) / 4;
     for (int idx = threadIdx.x; idx < KT4 * 64; idx += blockDim.x) {
         const int k4 = idx >> 6, l = idx & 63, c = l & 15, g = l >> 4;
+        const int ur = kX2 ? (c & 7) : c;
         uint32_t v = 0x7f7f7f7fu;
-        if (c < nrows) {
-            const int r = row_src(c);
-            if (r >= 0) v = *reinterpret_cast<const uint32_t*>(qs + (size_t)r * scale_pitch(K) + k4 * 16 + g * 4);
+        if (ur < nrows) {
+            const int r = row_src(ur);
+            const uint8_t* plane = (kX2 && c >= 8) ? qs2 : qs;
+            if (r >= 0) v = *reinterpret_cast<const uint32_t*>(plane + (size_t)r * spitch + k4 * 16 + g * 4);
         }
         bsc[idx] = v;
     }
+}
+
+// Two-term activations: lanes c and c ^ 8 of a 16-lane row hold the partial results of the same unit row.
+__device__ __forceinline__ void join_terms(v4f (&acc)[4]) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[t][v] += __shfl_xor(acc[t][v], 8, 64);
 }
 
 struct MfmaArgs {
@@ -247,10 +268,9 @@ __device__ __forceinline__ bool unit_block_work(const MfmaArgs& a, int groups, i
 // gate/up GEMM + clamped SwiGLU + e4m3-per-32 quantisation of the result.
 // grid: unit_block_work over groups = ceil(items / WAVES) item groups; wave w of item group ig owns item
 // ig*WAVES + w of the unit's expert.
-template <int WAVES, bool kKeep>
-__device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, const uint8_t* __restrict__ xq,
-                                             const uint8_t* __restrict__ xs, const int32_t* __restrict__ gather_src,
-                                             uint8_t* __restrict__ act_q, uint8_t* __restrict__ act_s,
+template <int WAVES, bool kKeep, bool kX2>
+__device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& xin,
+                                             const int32_t* __restrict__ gather_src, const ActPlanes& act,
                                              unsigned char* lds_raw) {
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;   // tables from an uninitialised workspace must not cause a fault
@@ -277,13 +297,14 @@ __device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, c
     const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
     StreamRegs regs;
     if (live) stream_load_group<kKeep>(regs, wp, sp, KT, lane, 0, 0);   // weights fly while the activations are staged
-    fill_b_operand(xq, xs, H, nrows, row_src, bq, bsc);
+    fill_b_operand<kX2>(xin.q, xin.s, xin.q2, xin.s2, H, (size_t)H, scale_pitch(H), nrows, row_src, bq, bsc);
     __syncthreads();
     if (!live) return;
     v4f acc[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
     stream_item<kKeep>(regs, wp, sp, KT, bq, bsc, lane, acc);
+    if constexpr (kX2) join_terms(acc);
 
     // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
     float r0[4], r1[4];
@@ -297,37 +318,56 @@ __device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, c
     amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
     const int c = lane & 15, g = lane >> 4;
-    if (c < nrows) {
-        const uint32_t sb = block_scale_e8m0(amax);
-        const float inv = u2f((254u - sb) << 23);
-        const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
-        const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
-        uint8_t* dst = act_q + (size_t)(row0 + c) * a.act_ld + (size_t)item * 32 + g * 4;
+    const int ur = kX2 ? (c & 7) : c;
+    const uint32_t sb = block_scale_e8m0(amax);
+    const float inv = u2f((254u - sb) << 23);
+    uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
+    uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
+    uint8_t* dq = act.q;
+    uint8_t* ds = act.s;
+    uint32_t sbo = sb;
+    if constexpr (kX2) {
+        // second term: the same quantiser on what the first leaves over; lanes c >= 8 store it, lanes c < 8 the first
+        const float sc = u2f(sb << 23);
+        float amax2 = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            r0[v] = fadd(r0[v], -fmul(e4m3_decode((p0 >> (8 * v)) & 0xffu), sc));
+            r1[v] = fadd(r1[v], -fmul(e4m3_decode((p1 >> (8 * v)) & 0xffu), sc));
+            amax2 = fmaxf(amax2, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+        }
+        amax2 = fmaxf(amax2, __shfl_xor(amax2, 16, 64));
+        amax2 = fmaxf(amax2, __shfl_xor(amax2, 32, 64));
+        const uint32_t sb2 = block_scale_e8m0(amax2);
+        const float inv2 = u2f((254u - sb2) << 23);
+        const uint32_t t0 = e4m3_encode4_hw(r0[0] * inv2, r0[1] * inv2, r0[2] * inv2, r0[3] * inv2);
+        const uint32_t t1 = e4m3_encode4_hw(r1[0] * inv2, r1[1] * inv2, r1[2] * inv2, r1[3] * inv2);
+        if (c >= 8) { p0 = t0; p1 = t1; sbo = sb2; dq = act.q2; ds = act.s2; }
+    }
+    if (ur < nrows) {
+        uint8_t* dst = dq + (size_t)(row0 + ur) * a.act_ld + (size_t)item * 32 + g * 4;
         *reinterpret_cast<uint32_t*>(dst) = p0;
         *reinterpret_cast<uint32_t*>(dst + 16) = p1;
-        if (g == 0) act_s[(size_t)(row0 + c) * scale_pitch(a.act_ld) + scale_pos(item)] = (uint8_t)sb;
+        if (g == 0) ds[(size_t)(row0 + ur) * scale_pitch(a.act_ld) + scale_pos(item)] = (uint8_t)sbo;
     }
 }
 
-template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ xq,
-                                                                  const uint8_t* __restrict__ xs,
+template <int WAVES, bool kX2>
+__global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, int groups, ActPlanes xin,
                                                                   const int32_t* __restrict__ gather_src,
-                                                                  uint8_t* __restrict__ act_q,
-                                                                  uint8_t* __restrict__ act_s) {
+                                                                  ActPlanes act) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig, ne;
     if (!unit_block_work(a, groups, u, ig, ne)) return;
     // an expert with several units: its weights are wanted again by the blocks that follow on this XCD
-    if (ne > 1) gate_up_unit<WAVES, true>(a, u, ig, xq, xs, gather_src, act_q, act_s, lds_raw);
-    else gate_up_unit<WAVES, false>(a, u, ig, xq, xs, gather_src, act_q, act_s, lds_raw);
+    if (ne > 1) gate_up_unit<WAVES, true, kX2>(a, u, ig, xin, gather_src, act, lds_raw);
+    else gate_up_unit<WAVES, false, kX2>(a, u, ig, xin, gather_src, act, lds_raw);
 }
 
 // down GEMM: y[row][h] for the unit's rows.  grid: unit_block_work over groups = ceil(items / (WAVES*IPW)); item =
 // 64 rows of H.
-template <int WAVES, int IPW, bool kKeep>
-__device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, const uint8_t* __restrict__ act_q,
-                                          const uint8_t* __restrict__ act_s, float* __restrict__ y,
+template <int WAVES, int IPW, bool kKeep, bool kX2>
+__device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& act, float* __restrict__ y,
                                           unsigned char* lds_raw) {
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
@@ -347,22 +387,8 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
                           reinterpret_cast<const u4v*>(sb) + (size_t)item0 * KT4 * 64, KT, lane, 0, 0);
     }
     // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
-    {
-        const int chunks = inter / 16;
-        for (int idx = threadIdx.x; idx < nrows * chunks; idx += blockDim.x) {
-            const int c = idx / chunks, j = idx % chunks;
-            u4v v = *reinterpret_cast<const u4v*>(act_q + (size_t)(row0 + c) * a.act_ld + (size_t)j * 16);
-            const int k = j * 16, kt = k >> 7, within = k & 127;
-            bq[(kt * 2 + (within >> 6)) * 64 + ((within & 63) >> 4) * 16 + c] = v;
-        }
-        for (int idx = threadIdx.x; idx < KT4 * 64; idx += blockDim.x) {
-            const int k4 = idx >> 6, l = idx & 63, c = l & 15, g = l >> 4;
-            uint32_t v = 0x7f7f7f7fu;
-            if (c < nrows)
-                v = *reinterpret_cast<const uint32_t*>(act_s + (size_t)(row0 + c) * scale_pitch(a.act_ld) + k4 * 16 + g * 4);
-            bsc[idx] = v;
-        }
-    }
+    fill_b_operand<kX2>(act.q, act.s, act.q2, act.s2, inter, (size_t)a.act_ld, scale_pitch(a.act_ld), nrows,
+                        [&](int c) { return row0 + c; }, bq, bsc);
     __syncthreads();
     const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
     const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
@@ -378,7 +404,8 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
         stream_item<kKeep>(regs, wp, sp, KT, bq, bsc, lane, acc);
-        if (c < nrows) {
+        if constexpr (kX2) join_terms(acc);
+        if (c < nrows && (!kX2 || c < 8)) {
             float* dst = y + (size_t)(row0 + c) * H + (size_t)item * 64 + g * 4;
 #pragma unroll
             for (int t = 0; t < 4; ++t)
@@ -387,15 +414,14 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
     }
 }
 
-template <int WAVES, int IPW>
-__global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, int groups, const uint8_t* __restrict__ act_q,
-                                                               const uint8_t* __restrict__ act_s,
+template <int WAVES, int IPW, bool kX2>
+__global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, int groups, ActPlanes act,
                                                                float* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig, ne;
     if (!unit_block_work(a, groups, u, ig, ne)) return;
-    if (ne > 1) down_unit<WAVES, IPW, true>(a, u, ig, act_q, act_s, y, lds_raw);
-    else down_unit<WAVES, IPW, false>(a, u, ig, act_q, act_s, y, lds_raw);
+    if (ne > 1) down_unit<WAVES, IPW, true, kX2>(a, u, ig, act, y, lds_raw);
+    else down_unit<WAVES, IPW, false, kX2>(a, u, ig, act, y, lds_raw);
 }
 
 
@@ -710,63 +736,81 @@ static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int
 }
 
 // k_start / k_stop (may be null): events that bracket the kernel itself on the device, not the launch.
-int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
-                        int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
-                        hipStream_t st, hipEvent_t k_start, hipEvent_t k_stop) {
+int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& xin, int n,
+                        const int32_t* gather_src, const UnitTables& units, const ActPlanes& act, hipStream_t st,
+                        hipEvent_t k_start, hipEvent_t k_stop) {
     MfmaArgs a = make_args(s, packed, n, units, false);
     const int imax = a.act_ld;
+    const bool x2 = xin.q2 != nullptr;
+    if (x2 != (act.q2 != nullptr)) return FERRITE_ERR_INVALID_ARG;
     if (units.unit_rows_cap == PF_ROWS) {
+        if (x2) return FERRITE_ERR_INVALID_ARG;   // the 128-row kernels take one-term activations
         const int groups = (imax / 32 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
         int rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES);
         if (rc) return rc;
         hipExtLaunchKernelGGL(gate_up_prefill_kernel, dim3(blocks), dim3(PF_WAVES * 64), (uint32_t)PF_LDS_BYTES, st, k_start,
-                              k_stop, 0, a, groups, xq, xs, gather_src, act_q, act_s);
+                              k_stop, 0, a, groups, xin.q, xin.s, gather_src, act.q, act.s);
         return check_launch("gate_up_prefill");
     }
-    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
+    if (units.unit_rows_cap != (x2 ? 8 : 16)) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = (size_t)s.hidden * 16 + (size_t)((s.hidden / 128 + 3) / 4) * 256;
-    int rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES>>::ensure(lds);
-    if (rc) return rc;
     const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
     const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-    hipExtLaunchKernelGGL(gate_up_mfma_kernel<GU_WAVES>, dim3(blocks), dim3(GU_WAVES * 64), (uint32_t)lds, st, k_start,
-                          k_stop, 0, a, groups, xq, xs, gather_src, act_q, act_s);
+    int rc;
+    if (x2) {
+        if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true>>::ensure(lds))) return rc;
+        hipExtLaunchKernelGGL((gate_up_mfma_kernel<GU_WAVES, true>), dim3(blocks), dim3(GU_WAVES * 64), (uint32_t)lds, st,
+                              k_start, k_stop, 0, a, groups, xin, gather_src, act);
+    } else {
+        if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false>>::ensure(lds))) return rc;
+        hipExtLaunchKernelGGL((gate_up_mfma_kernel<GU_WAVES, false>), dim3(blocks), dim3(GU_WAVES * 64), (uint32_t)lds, st,
+                              k_start, k_stop, 0, a, groups, xin, gather_src, act);
+    }
     return check_launch("gate_up_mfma");
 }
 
-int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
-                     int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
+int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& act, int n,
+                     const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
     MfmaArgs a = make_args(s, packed, n, units, true);
+    const bool x2 = act.q2 != nullptr;
     if (units.unit_rows_cap == PF_ROWS) {
+        if (x2) return FERRITE_ERR_INVALID_ARG;
         const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
         int rc;
         if (y_dtype == FERRITE_DT_BF16) {
             if ((rc = LdsLimit<&down_prefill_kernel<uint16_t>>::ensure(PF_LDS_BYTES))) return rc;
-            down_prefill_kernel<uint16_t><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<uint16_t*>(y));
+            down_prefill_kernel<uint16_t><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act.q, act.s, static_cast<uint16_t*>(y));
         } else {
             if ((rc = LdsLimit<&down_prefill_kernel<float>>::ensure(PF_LDS_BYTES))) return rc;
-            down_prefill_kernel<float><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
+            down_prefill_kernel<float><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act.q, act.s, static_cast<float*>(y));
         }
         return check_launch("down_prefill");
     }
-    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
+    if (units.unit_rows_cap != (x2 ? 8 : 16)) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = (size_t)a.act_ld * 16 + (size_t)((a.act_ld / 128 + 3) / 4) * 256;
-    int rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW>>::ensure(lds);
-    if (rc) return rc;
     const int items = s.hidden / 64;
     const int groups = (items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW);
     const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
     if (y_dtype != FERRITE_DT_F32) return FERRITE_ERR_INVALID_ARG;
-    down_mfma_kernel<DN_WAVES, DN_IPW><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act_q, act_s, static_cast<float*>(y));
+    int rc;
+    if (x2) {
+        if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(lds))) return rc;
+        down_mfma_kernel<DN_WAVES, DN_IPW, true><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, static_cast<float*>(y));
+    } else {
+        if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(lds))) return rc;
+        down_mfma_kernel<DN_WAVES, DN_IPW, false><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, static_cast<float*>(y));
+    }
     return check_launch("down_mfma");
 }
 
 int warmup_experts_mfma() {
     int rc;
-    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES>>::ensure(kLdsCap))) return rc;
-    if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES))) return rc;
     if ((rc = LdsLimit<&down_prefill_kernel<uint16_t>>::ensure(PF_LDS_BYTES))) return rc;
     return LdsLimit<&down_prefill_kernel<float>>::ensure(PF_LDS_BYTES);

@@ -31,17 +31,24 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t* __res
     }
 }
 
-// One thread quantises one block of 32 consecutive values of a row.
+// One thread quantises one block of 32 consecutive values of a row; with q2 / scale2, a second term from the
+// residual of the first (quant_block32_x2).
 // operand_order: scales go to scale_pos() within rows of scale_pitch(cols) bytes instead of row-major.
 template <typename XT>
 __global__ __launch_bounds__(256) void act_quant_kernel(const XT* __restrict__ x, int64_t nblocks, int bpr,
                                                         int operand_order, uint8_t* __restrict__ q,
-                                                        uint8_t* __restrict__ scale) {
+                                                        uint8_t* __restrict__ scale, uint8_t* __restrict__ q2,
+                                                        uint8_t* __restrict__ scale2) {
     int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nblocks) return;
-    const uint8_t sb = (uint8_t)quant_block32(x + b * 32, q + b * 32);
-    if (operand_order) scale[(b / bpr) * scale_pitch(bpr * 32) + scale_pos((int)(b % bpr))] = sb;
-    else scale[b] = sb;
+    const int64_t at = operand_order ? (b / bpr) * scale_pitch(bpr * 32) + scale_pos((int)(b % bpr)) : b;
+    if (q2) {
+        const uint32_t sb = quant_block32_x2(x + b * 32, q + b * 32, q2 + b * 32);
+        scale[at] = (uint8_t)(sb & 0xffu);
+        scale2[at] = (uint8_t)(sb >> 8);
+    } else {
+        scale[at] = (uint8_t)quant_block32(x + b * 32, q + b * 32);
+    }
 }
 
 // Weights to MXFP4, one thread per block of 32 consecutive values of a row (quant.rs:217-238 with the
@@ -102,16 +109,16 @@ __global__ __launch_bounds__(256) void mxfp4_quant_kernel(const XT* __restrict__
     scale[b] = (uint8_t)sb;
 }
 
-int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, int operand_order,
-                     hipStream_t st) {
-    if (rows < 0 || cols < 0 || cols % 32 != 0) return FERRITE_ERR_INVALID_ARG;
+int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, uint8_t* q2,
+                     uint8_t* scale2, int operand_order, hipStream_t st) {
+    if (rows < 0 || cols < 0 || cols % 32 != 0 || (q2 == nullptr) != (scale2 == nullptr)) return FERRITE_ERR_INVALID_ARG;
     int64_t nblocks = rows * (cols / 32);
     if (nblocks == 0) return FERRITE_OK;
     unsigned grid = (unsigned)((nblocks + 255) / 256);
     if (x_dtype == FERRITE_DT_F32)
-        act_quant_kernel<float><<<grid, 256, 0, st>>>((const float*)x, nblocks, cols / 32, operand_order, q, scale);
+        act_quant_kernel<float><<<grid, 256, 0, st>>>((const float*)x, nblocks, cols / 32, operand_order, q, scale, q2, scale2);
     else if (x_dtype == FERRITE_DT_BF16)
-        act_quant_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)x, nblocks, cols / 32, operand_order, q, scale);
+        act_quant_kernel<uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)x, nblocks, cols / 32, operand_order, q, scale, q2, scale2);
     else
         return FERRITE_ERR_INVALID_ARG;
     return check_launch("act_quant");
@@ -153,5 +160,14 @@ extern "C" int ferrite_act_quant_fp8(const void* x, int x_dtype, int64_t rows, i
                                      ferrite_stream_t stream) {
     if (rows > 0 && cols > 0 && (!x || !q || !scale)) return FERRITE_ERR_INVALID_ARG;
     if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(q) & 15)) return FERRITE_DECLINED;
-    return launch_act_quant(x, x_dtype, rows, cols, q, scale, 0, as_stream(stream));
+    return launch_act_quant(x, x_dtype, rows, cols, q, scale, nullptr, nullptr, 0, as_stream(stream));
+}
+
+extern "C" int ferrite_act_quant_fp8_x2(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q1, uint8_t* scale1,
+                                        uint8_t* q2, uint8_t* scale2, ferrite_stream_t stream) {
+    if (rows > 0 && cols > 0 && (!x || !q1 || !scale1 || !q2 || !scale2)) return FERRITE_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(q1) & 15) ||
+        (reinterpret_cast<uintptr_t>(q2) & 15))
+        return FERRITE_DECLINED;
+    return launch_act_quant(x, x_dtype, rows, cols, q1, scale1, q2, scale2, 0, as_stream(stream));
 }

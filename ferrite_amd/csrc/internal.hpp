@@ -70,6 +70,12 @@ struct LdsLimit {
 int warmup_route();
 int warmup_experts_mfma();
 
+// Activation buffers of the expert GEMMs: e4m3 codes and operand-order scales, one plane, or two for two-term
+// activations (q2 / s2 null otherwise).
+struct ActPlanes {
+    uint8_t *q, *s, *q2, *s2;
+};
+
 // route.hip
 int launch_matmul_exact(const void* x, int x_dtype, const float* w, const float* bias, float* out, int n, int k,
                         int o, hipStream_t st);
@@ -81,7 +87,7 @@ int check_routing_params(int e, int topk, int n_group, int topk_group);
 size_t perm_scratch_bytes(int n_tokens, int n_experts);   // masks + offsets of the three-phase permutation
 bool head_supported(int n, int H, int E);
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
-                    int n, float* logits, float* probs, float* ids_f32, int32_t* ids, uint8_t* xq, uint8_t* xs,
+                    int n, float* logits, float* probs, float* ids_f32, int32_t* ids, const ActPlanes& xq,
                     int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
                     int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, hipStream_t st);
 int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
@@ -107,11 +113,11 @@ struct PackedLayout {
     size_t total;
 };
 PackedLayout packed_layout(const ferrite_moe_shape& s);
-int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* xq, const uint8_t* xs,
-                        int n, const int32_t* gather_src, const UnitTables& units, uint8_t* act_q, uint8_t* act_s,
-                        hipStream_t st, hipEvent_t k_start = nullptr, hipEvent_t k_stop = nullptr);
-int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const uint8_t* act_q, const uint8_t* act_s,
-                     int n, const UnitTables& units, void* y, int y_dtype, hipStream_t st);
+int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& xin, int n,
+                        const int32_t* gather_src, const UnitTables& units, const ActPlanes& act, hipStream_t st,
+                        hipEvent_t k_start = nullptr, hipEvent_t k_stop = nullptr);
+int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& act, int n,
+                     const UnitTables& units, void* y, int y_dtype, hipStream_t st);
 
 // block_ops.hip
 int launch_rmsnorm(const float* x, const float* w, float eps, float* out, int n, int dim, hipStream_t st);
@@ -119,7 +125,8 @@ int launch_hc_post(const float* x, const float* residual, const float* post, con
                    int nh, int h, hipStream_t st);
 
 // formats.hip
-int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, int operand_order,
-                     hipStream_t st);
+// q2 / scale2 (both or neither): the second term of a two-term quantisation, from the residual of the first.
+int launch_act_quant(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale, uint8_t* q2,
+                     uint8_t* scale2, int operand_order, hipStream_t st);
 
 }  // namespace fe

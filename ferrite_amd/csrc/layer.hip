@@ -33,7 +33,7 @@ int check_launch(const char* what) {
 struct Workspace {
     size_t logits, probs, ids_f32, ids, counts, starts, perm_map, gather_src, active, n_active;
     size_t unit_expert, unit_row0, unit_rows, unit_first, unit_count, n_units, perm_scratch, perm_scratch_bytes, counters;
-    size_t xq, xs, act, act_s, y;
+    size_t xq, xs, xq2, xs2, act, act_s, act2, act_s2, y;
     size_t total;
     int max_units, rows, unit_cap;
 };
@@ -70,6 +70,8 @@ int raise_lds_limit(const void* kernel, size_t bytes, std::atomic<size_t>* raise
     return FERRITE_OK;
 }
 
+static bool is_mfma_mode(int mode) { return mode == FERRITE_MODE_MFMA_FP8 || mode == FERRITE_MODE_MFMA_FP8_X2; }
+
 static size_t bump(size_t& off, size_t bytes) {
     size_t at = off;
     off = (off + bytes + 255) / 256 * 256;
@@ -82,7 +84,9 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     const int has_shared = s.shared_inter > 0;
     const size_t act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
     w.rows = (int)(nk + (has_shared ? n : 0));
-    w.unit_cap = mode == FERRITE_MODE_MFMA_FP8 ? unit_rows_for(n, s.topk, s.n_experts) : 16;
+    // two-term activations: 8-row units (the two terms of a row share one 16-column operand)
+    w.unit_cap = mode == FERRITE_MODE_MFMA_FP8 ? unit_rows_for(n, s.topk, s.n_experts)
+                                               : (mode == FERRITE_MODE_MFMA_FP8_X2 ? 8 : 16);
     w.max_units = max_units_for(n, s.topk, s.n_experts, has_shared, w.unit_cap);
     size_t off = 0;
     w.counters = bump(off, ((size_t)n + 1) * 4);   // first: ferrite_moe_layer_workspace_init clears it
@@ -104,11 +108,18 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     w.n_units = bump(off, 4);
     w.perm_scratch_bytes = perm_scratch_bytes(n, s.n_experts);
     w.perm_scratch = bump(off, w.perm_scratch_bytes);
-    if (mode == FERRITE_MODE_MFMA_FP8) {
+    if (is_mfma_mode(mode)) {
+        const size_t xs_row = ((H / 128 + 3) / 4) * 16, as_row = ((act_ld / 128 + 3) / 4) * 16;
         w.xq = bump(off, (size_t)n * H);
-        w.xs = bump(off, (size_t)n * (((H / 128 + 3) / 4) * 16));
+        w.xs = bump(off, (size_t)n * xs_row);
         w.act = bump(off, (size_t)w.rows * act_ld);
-        w.act_s = bump(off, (size_t)w.rows * (((act_ld / 128 + 3) / 4) * 16));
+        w.act_s = bump(off, (size_t)w.rows * as_row);
+        if (mode == FERRITE_MODE_MFMA_FP8_X2) {
+            w.xq2 = bump(off, (size_t)n * H);
+            w.xs2 = bump(off, (size_t)n * xs_row);
+            w.act2 = bump(off, (size_t)w.rows * act_ld);
+            w.act_s2 = bump(off, (size_t)w.rows * as_row);
+        }
     } else {
         w.act = bump(off, (size_t)w.rows * act_ld * 4);
     }
@@ -122,10 +133,11 @@ static int check_shape(const ferrite_moe_shape* s, int n, int mode) {
     if (s->hidden <= 0 || s->n_experts <= 0 || s->topk <= 0 || s->topk > s->n_experts || s->inter <= 0 ||
         s->shared_inter < 0)
         return FERRITE_ERR_INVALID_ARG;
-    if (mode != FERRITE_MODE_F32_CHECK && mode != FERRITE_MODE_MFMA_FP8) return FERRITE_ERR_INVALID_ARG;
+    if (mode != FERRITE_MODE_F32_CHECK && !is_mfma_mode(mode)) return FERRITE_ERR_INVALID_ARG;
     if (s->hidden % 32 || s->inter % 32 || s->shared_inter % 32) return FERRITE_ERR_INVALID_ARG;
-    if (mode == FERRITE_MODE_MFMA_FP8 && (s->hidden % 128 || s->inter % 128 || s->shared_inter % 128))
-        return FERRITE_DECLINED;
+    if (is_mfma_mode(mode) && (s->hidden % 128 || s->inter % 128 || s->shared_inter % 128)) return FERRITE_DECLINED;
+    // two-term activations exist for the weight-streaming kernels only (decode-sized batches)
+    if (mode == FERRITE_MODE_MFMA_FP8_X2 && (long)n * s->topk >= 48L * s->n_experts) return FERRITE_DECLINED;
     if (n > 65535) return FERRITE_DECLINED;   // token index on grid.y of several kernels: split the batch
     // the routing kernels' own limits, for the fused head and the separate launches alike
     return check_routing_params(s->n_experts, s->topk, s->n_group, s->topk_group);
@@ -247,14 +259,16 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     int32_t* perm_map = reinterpret_cast<int32_t*>(b + w.perm_map);
     int32_t* gather_src = reinterpret_cast<int32_t*>(b + w.gather_src);
     void* y = b + w.y;
-    const int y_dtype = mode == FERRITE_MODE_MFMA_FP8 ? y_dtype_for(w.unit_cap) : FERRITE_DT_F32;
+    const int y_dtype = is_mfma_mode(mode) ? y_dtype_for(w.unit_cap) : FERRITE_DT_F32;
+    const bool x2 = mode == FERRITE_MODE_MFMA_FP8_X2;
+    auto at = [&](size_t off) { return reinterpret_cast<uint8_t*>(b + off); };
+    const ActPlanes xq = is_mfma_mode(mode) ? ActPlanes{at(w.xq), at(w.xs), x2 ? at(w.xq2) : nullptr, x2 ? at(w.xs2) : nullptr}
+                                            : ActPlanes{nullptr, nullptr, nullptr, nullptr};
 
     UnitTables units{reinterpret_cast<int32_t*>(b + w.unit_expert), reinterpret_cast<int32_t*>(b + w.unit_row0),
                      reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.unit_first),
                      reinterpret_cast<int32_t*>(b + w.unit_count), reinterpret_cast<int32_t*>(b + w.n_units), w.unit_cap,
                      w.max_units};
-    uint8_t* xq = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xq) : nullptr;
-    uint8_t* xs = mode == FERRITE_MODE_MFMA_FP8 ? reinterpret_cast<uint8_t*>(b + w.xs) : nullptr;
     if ((rc = mark(ev, 0, st))) return rc;
     const bool fused_head = packed != nullptr && head_supported(n, s.hidden, s.n_experts);
     if (fused_head) {
@@ -262,7 +276,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         PackedLayout L = packed_layout(s);
         const int fuse_perm = 1;   // the block that routes the last token builds the tables
         if ((rc = launch_moe_head(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), wts->router_bias, s,
-                                  n, logits, probs, ids_f32, ids, xq, xs, reinterpret_cast<int32_t*>(b + w.counters),
+                                  n, logits, probs, ids_f32, ids, xq, reinterpret_cast<int32_t*>(b + w.counters),
                                   reinterpret_cast<int32_t*>(b + w.counts), reinterpret_cast<int32_t*>(b + w.starts),
                                   perm_map, gather_src, reinterpret_cast<int32_t*>(b + w.active),
                                   reinterpret_cast<int32_t*>(b + w.n_active), &units, fuse_perm, st)))
@@ -304,8 +318,8 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                              b + w.perm_scratch, w.perm_scratch_bytes, &units, has_shared, st)))
         return rc;
     if ((rc = mark(ev, 3, st))) return rc;
-    if (xq) {
-        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq, xs, 1, st))) return rc;
+    if (xq.q) {
+        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq.q, xq.s, xq.q2, xq.s2, 1, st))) return rc;
     }
     if ((rc = mark(ev, 4, st))) return rc;
     }
@@ -316,14 +330,13 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         if ((rc = mark(ev, 5, st))) return rc;
         if ((rc = launch_down_f32(s, *wts, act, n, ids, gather_src, static_cast<float*>(y), st))) return rc;
     } else {
-        uint8_t* act_q = reinterpret_cast<uint8_t*>(b + w.act);
-        uint8_t* act_s = reinterpret_cast<uint8_t*>(b + w.act_s);
-        if ((rc = launch_gate_up_mfma(s, packed, xq, xs, n, gather_src, units, act_q, act_s, st,
+        const ActPlanes act{at(w.act), at(w.act_s), x2 ? at(w.act2) : nullptr, x2 ? at(w.act_s2) : nullptr};
+        if ((rc = launch_gate_up_mfma(s, packed, xq, n, gather_src, units, act, st,
                                       ev ? static_cast<hipEvent_t>(ev[8]) : nullptr,
                                       ev ? static_cast<hipEvent_t>(ev[9]) : nullptr)))
             return rc;
         if ((rc = mark(ev, 5, st))) return rc;
-        if ((rc = launch_down_mfma(s, packed, act_q, act_s, n, units, y, y_dtype, st))) return rc;
+        if ((rc = launch_down_mfma(s, packed, act, n, units, y, y_dtype, st))) return rc;
     }
     if ((rc = mark(ev, 6, st))) return rc;
     // 6. weighted combine in slot order + shared expert (exec/lib.rs:1154-1164)

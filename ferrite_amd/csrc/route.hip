@@ -560,7 +560,7 @@ struct HeadArgs {
     float scaling;
     float *logits, *probs, *ids_f32;
     int32_t* ids;
-    uint8_t *xq, *xs;     // may be NULL: no quantisation blocks are launched then
+    ActPlanes xq;         // q may be NULL: no quantisation blocks are launched then; q2 set: two-term
     int32_t* counters;    // [1 + n]
     int fuse_perm;        // the block that routes the last token also builds the permutation; else a separate launch does
     PermArgs perm;
@@ -732,9 +732,16 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
             const int t = t0 + ti;
             if (t >= a.n) break;
             const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
-            for (int b = tid; b < H / 32; b += 512)
-                a.xs[(size_t)t * scale_pitch(H) + scale_pos(b)] =
-                    (uint8_t)quant_block32(xrow + b * 32, a.xq + (size_t)t * H + b * 32);
+            for (int b = tid; b < H / 32; b += 512) {
+                const size_t at = (size_t)t * scale_pitch(H) + scale_pos(b), qo = (size_t)t * H + b * 32;
+                if (a.xq.q2) {
+                    const uint32_t sb = quant_block32_x2(xrow + b * 32, a.xq.q + qo, a.xq.q2 + qo);
+                    a.xq.s[at] = (uint8_t)(sb & 0xffu);
+                    a.xq.s2[at] = (uint8_t)(sb >> 8);
+                } else {
+                    a.xq.s[at] = (uint8_t)quant_block32(xrow + b * 32, a.xq.q + qo);
+                }
+            }
         }
         return;
     }
@@ -856,7 +863,7 @@ static int launch_head_t(const HeadArgs& a, int quant, size_t lds, hipStream_t s
 }
 
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
-                    int n, float* logits, float* probs, float* ids_f32, int32_t* ids, uint8_t* xq, uint8_t* xs,
+                    int n, float* logits, float* probs, float* ids_f32, int32_t* ids, const ActPlanes& xq,
                     int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
                     int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, hipStream_t st) {
     if (!head_supported(n, s.hidden, s.n_experts)) return FERRITE_DECLINED;
@@ -865,7 +872,7 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
     a.n = n; a.H = s.hidden; a.E = s.n_experts; a.Epad = (s.n_experts + 63) / 64 * 64; a.topk = s.topk;
     a.n_group = (s.n_group > 1 && s.topk_group < s.n_group) ? s.n_group : 1;
     a.topk_group = s.topk_group; a.scaling = s.routed_scaling;
-    a.logits = logits; a.probs = probs; a.ids_f32 = ids_f32; a.ids = ids; a.xq = xq; a.xs = xs; a.counters = counters;
+    a.logits = logits; a.probs = probs; a.ids_f32 = ids_f32; a.ids = ids; a.xq = xq; a.counters = counters;
     a.fuse_perm = fuse_perm;
     PermArgs& p = a.perm;
     p.ids = ids; p.n = n; p.topk = s.topk; p.n_experts = s.n_experts;
@@ -877,8 +884,8 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
         p.n_units = units->n_units; p.unit_cap = units->unit_rows_cap; p.max_units = units->max_units;
     }
     const size_t lds = head_lds_bytes(n, s.hidden, s.n_experts, true);
-    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, xq ? 1 : 0, lds, st);
-    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, true>(a, xq ? 1 : 0, lds, st);
+    if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, xq.q ? 1 : 0, lds, st);
+    if (x_dtype == FERRITE_DT_BF16) return launch_head_t<uint16_t, true>(a, xq.q ? 1 : 0, lds, st);
     return FERRITE_ERR_INVALID_ARG;
 }
 

@@ -41,6 +41,11 @@ extern "C" {
 /* layer arithmetic modes */
 #define FERRITE_MODE_F32_CHECK 0   /* f32 activations, weights dequantised exactly, f32 FMA dot products */
 #define FERRITE_MODE_MFMA_FP8 1    /* activations quantised e4m3 per 32 (e8m0 scale), block-scaled MFMA */
+#define FERRITE_MODE_MFMA_FP8_X2 2 /* the same with two-term activations: x ~ q1*s1 + q2*s2, the second term being the
+                                    * e4m3-per-32 quantisation of what the first leaves over (about 8 significant
+                                    * bits, bf16-class).  Decode-sized batches only (n*topk < 48*n_experts), where
+                                    * the matrix cores idle behind the weight stream and the second term is free;
+                                    * larger batches return FERRITE_DECLINED (use FERRITE_MODE_MFMA_FP8). */
 
 typedef void* ferrite_stream_t;
 
@@ -113,6 +118,13 @@ int ferrite_mxfp4_quant(const void* x, int x_dtype, int64_t rows, int64_t cols, 
  * q [rows, cols] e4m3 codes, scale [rows, cols/32] e8m0 bytes (2^(b-127)). */
 int ferrite_act_quant_fp8(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q, uint8_t* scale,
                           ferrite_stream_t stream);
+
+/* The two-term form of ferrite_act_quant_fp8 that FERRITE_MODE_MFMA_FP8_X2 feeds the matrix cores with: q1 / scale1
+ * as above, then q2 / scale2 = the same quantiser applied to the residual x - decode(q1) * scale1 (one f32
+ * multiply by the power-of-two scale and one f32 subtraction per value).  No counterpart in the reference, whose
+ * device path quantises once (dsv41_quant_fp8, crates/ferrite-models/src/dsv41/kernels.rs:97-108). */
+int ferrite_act_quant_fp8_x2(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q1, uint8_t* scale1,
+                             uint8_t* q2, uint8_t* scale2, ferrite_stream_t stream);
 
 /* ---- the fused layer: the counterpart of CudaBackend::moe_layer_dev (cuda.rs:5604-6142) for MXFP4 experts
  *      with group-limited routing; caller = Engine::moe_ffn (crates/ferrite-exec/src/lib.rs:1083-1166) ---- */
@@ -189,7 +201,8 @@ typedef struct ferrite_moe_workspace_view {
 
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
 /* Rows per unit (the token tile of the expert GEMMs) a layer call with these arguments uses: 16 = weights streamed
- * once per unit (decode-sized batches), 128 = both operands tiled through LDS (prefill-sized batches); 0 for an
+ * once per unit (decode-sized batches; 8 with two-term activations, whose two terms share the 16 operand columns),
+ * 128 = both operands tiled through LDS (prefill-sized batches); 0 for an
  * unsupported shape.  The choice is a pure function of (shape, n, mode) and of the FERRITE_OVERRIDE_UNIT_ROWS
  * override, like the workspace layout that depends on it.
  * No counterpart in the reference, whose grouped GEMM has one tile shape (dsv41_moe.cu); informational. */
@@ -203,7 +216,7 @@ int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, int n, int 
                                      ferrite_moe_workspace_view* view_host);
 
 /* The layer.  x [n, H] (x_dtype), out [n, H] (out_dtype).  mode FERRITE_MODE_F32_CHECK reads `w` (checkpoint
- * layout) and requires f32 x; FERRITE_MODE_MFMA_FP8 reads `packed` and w->router_bias.  `packed` carries the
+ * layout) and requires f32 x; the FERRITE_MODE_MFMA_* modes read `packed` and w->router_bias.  `packed` carries the
  * router weight, so w->router_w may be NULL with it; the few shapes whose router falls back to the checkpoint
  * layout (very large hidden) then return FERRITE_ERR_INVALID_ARG.  n > 65535 and routing parameters outside
  * ferrite_moe_route's limits are refused up front (FERRITE_DECLINED / FERRITE_ERR_INVALID_ARG, as that op returns

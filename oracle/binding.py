@@ -67,6 +67,7 @@ def lib() -> C.CDLL:
         L.fo_act_quant_fp8.restype = None
         L.fo_act_quant_fp8.argtypes = [vp, C.c_size_t, C.c_int, C.c_int, vp, vp]
         L.fo_act_quant_fp4.restype = None
+        L.fo_act_quant_fp8_x2.argtypes = [vp, C.c_size_t, vp, vp, vp, vp]
         L.fo_act_quant_fp4.argtypes = [vp, C.c_size_t, C.c_int, C.c_int, vp, vp]
         L.fo_dequant_fp4_row32.restype = None
         L.fo_dequant_fp4_row32.argtypes = [vp, vp, C.c_size_t, C.c_size_t, vp]
@@ -125,6 +126,15 @@ def act_quant_fp8(x, block: int = 32, round_scale: bool = True):
     s = np.empty(x.size // block, np.float32)
     lib().fo_act_quant_fp8(_p(x), x.size, block, int(round_scale), _p(y), _p(s))
     return y, s
+
+
+def act_quant_fp8_x2(x):
+    """Two-term quantisation (block 32, power-of-two scales): (q1, s1, q2, s2) with x ~ dq1 + dq2."""
+    x = _f32(x).ravel()
+    q1, q2 = np.empty(x.size, np.uint8), np.empty(x.size, np.uint8)
+    s1, s2 = np.empty(x.size // 32, np.float32), np.empty(x.size // 32, np.float32)
+    lib().fo_act_quant_fp8_x2(_p(x), x.size, _p(q1), _p(s1), _p(q2), _p(s2))
+    return q1, s1, q2, s2
 
 
 def act_quant_fp4(x, block: int = 32, round_scale: bool = True):

@@ -475,6 +475,29 @@ static void qdq_row_fp8(const float* x, int len, float* dst, uint8_t* tmpq, floa
     for (int i = 0; i < len; ++i) dst[i] = fo_e4m3_decode(tmpq[i]) * tmps[i / 32];
 }
 
+/* Two-term form: q1/s1 = act_quant_fp8(x), q2/s2 = act_quant_fp8(x - decode(q1)*s1): x ~ dq1 + dq2.
+ * Not in the reference (its device path quantises once, kernels.rs:97-108): the composition of its quantiser with
+ * one f32 subtraction, stated here so that the device's two-term mode has a bit-level definition. */
+void fo_act_quant_fp8_x2(const float* x, size_t len, uint8_t* q1, float* s1, uint8_t* q2, float* s2) {
+    float* r = (float*)malloc(sizeof(float) * len);
+    fo_act_quant_fp8(x, len, 32, 1, q1, s1);
+    for (size_t i = 0; i < len; ++i) r[i] = x[i] - fo_e4m3_decode(q1[i]) * s1[i / 32];
+    fo_act_quant_fp8(r, len, 32, 1, q2, s2);
+    free(r);
+}
+
+/* quantise-dequantise one row through the two-term quantiser: dst = dq1 + dq2 (one f32 addition) */
+static void qdq_row_fp8_x2(const float* x, int len, float* dst) {
+    uint8_t* q1 = (uint8_t*)malloc((size_t)len * 2);
+    float* s1 = (float*)malloc(sizeof(float) * (size_t)(len / 32) * 2);
+    uint8_t* q2 = q1 + len;
+    float* s2 = s1 + len / 32;
+    fo_act_quant_fp8_x2(x, (size_t)len, q1, s1, q2, s2);
+    for (int i = 0; i < len; ++i)
+        dst[i] = fo_e4m3_decode(q1[i]) * s1[i / 32] + fo_e4m3_decode(q2[i]) * s2[i / 32];
+    free(q1); free(s1);
+}
+
 /* One expert applied to the rows listed in rows[] (token indices into xin).  y row r -> yout + r*H.
  * exec/lib.rs:1316-1332: gate = x.Wg^T, up = x.Wu^T, act = swiglu_limited([gate|up]), y = act.Wd^T. */
 static void expert_rows(const fo_moe_cfg* cfg, const float* xin, const int* rows, int m, const float* wg,
@@ -495,6 +518,7 @@ static void expert_rows(const fo_moe_cfg* cfg, const float* xin, const int* rows
             fo_swiglu_limited(gu, cfg->swiglu_limit, act, 1, inter);
             const float* a = act;
             if (cfg->act_mode == 1) { qdq_row_fp8(act, inter, actq, tq, ts); a = actq; }
+            else if (cfg->act_mode == 2) { qdq_row_fp8_x2(act, inter, actq); a = actq; }
             gemv_seq(a, wd, inter, H, ydst[r]);
         }
         free(gu); free(act); free(actq); free(tq); free(ts);
@@ -533,11 +557,14 @@ int fo_moe_ffn_mxfp4(const fo_moe_cfg* cfg, const fo_moe_weights* w, const float
     /* activations seen by the expert GEMMs */
     const float* xin = x;
     float* xq = NULL;
-    if (cfg->act_mode == 1) {
+    if (cfg->act_mode == 1 || cfg->act_mode == 2) {
         xq = (float*)malloc(sizeof(float) * (size_t)n * H);
         uint8_t* tq = (uint8_t*)malloc((size_t)H);
         float* ts = (float*)malloc(sizeof(float) * (size_t)(H / 32));
-        for (int r = 0; r < ns; ++r) qdq_row_fp8(x + (size_t)sel[r] * H, H, xq + (size_t)sel[r] * H, tq, ts);
+        for (int r = 0; r < ns; ++r) {
+            if (cfg->act_mode == 1) qdq_row_fp8(x + (size_t)sel[r] * H, H, xq + (size_t)sel[r] * H, tq, ts);
+            else qdq_row_fp8_x2(x + (size_t)sel[r] * H, H, xq + (size_t)sel[r] * H);
+        }
         free(tq); free(ts);
         xin = xq;
     }

@@ -54,6 +54,10 @@ float   fo_fast_pow2(int e);                          /* quant.rs:163-165 */
 float   fo_fast_round_scale(float amax);              /* quant.rs:169-174 */
 /* quant.rs:190-214: y[len] e4m3 codes, s[len/block] scales */
 void    fo_act_quant_fp8(const float* x, size_t len, int block, int round_scale, uint8_t* y, float* s);
+/* Two-term form (no reference counterpart: its quantiser composed with one f32 subtraction): q1/s1 =
+ * act_quant_fp8(x, 32, round_scale), q2/s2 = act_quant_fp8(x - decode(q1)*s1, 32, round_scale).
+ * PARITY UNPINNED by the reference; pinned by construction from fo_act_quant_fp8 (a NumPy composition in the tests). */
+void    fo_act_quant_fp8_x2(const float* x, size_t len, uint8_t* q1, float* s1, uint8_t* q2, float* s2);
 /* quant.rs:217-238: packed[len/2], s[len/block] */
 void    fo_act_quant_fp4(const float* x, size_t len, int block, int round_scale, uint8_t* packed, float* s);
 /* quant.rs:260-278: w [out, inn/2] u8, scale [out, inn/32] u8 -> dst [out, inn] f32 */
@@ -107,7 +111,10 @@ typedef struct {
     float swiglu_limit;
     int act_mode;        /* 0: f32 activations (CpuBackend proper);
                             1: x and the SwiGLU output are passed through act_quant_fp8(block 32,
-                               round_scale) and dequantised before each expert GEMM (quant.rs:201-214) */
+                               round_scale) and dequantised before each expert GEMM (quant.rs:201-214), where the
+                               reference's device chain quantises (dsv41_quant_fp8 in front of the first GEMM,
+                               dsv41_swiglu_limit_q after the SwiGLU: kernels.rs:97-108,586-598);
+                            2: the same two places through the two-term quantiser (fo_act_quant_fp8_x2) */
     int n_threads;       /* 1 = faithful single thread; >1 OpenMP over tokens/rows (never over k) */
 } fo_moe_cfg;
 

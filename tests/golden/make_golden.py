@@ -17,10 +17,11 @@ def main():
     inp = synth.make_inputs(synth.CONFIGS["c0"], seed=0)
     f32 = oracle.moe_ffn_mxfp4(inp, act_mode=0)
     fp8 = oracle.moe_ffn_mxfp4(inp, act_mode=1)
+    fp8x2 = oracle.moe_ffn_mxfp4(inp, act_mode=2)
     ids = f32["ids"].astype(np.int32)
     t = oracle.moe_permute(ids, inp.cfg.n_experts)
     np.savez_compressed(os.path.join(HERE, "c0_layer.npz"), ids=ids, probs=f32["probs"], logits=f32["logits"],
-                        out_f32=f32["out"], out_fp8act=fp8["out"], counts=t["counts"], starts=t["starts"],
+                        out_f32=f32["out"], out_fp8act=fp8["out"], out_fp8x2=fp8x2["out"], counts=t["counts"], starts=t["starts"],
                         perm_map=t["perm_map"], gather_src=t["gather_src"],
                         x_head=inp.x[0, :8], gate_w_head=inp.gate_w[0, 0, :8], gate_s_head=inp.gate_s[0, 0, :4])
     # format sweep tables: e4m3 decode of all 256 bytes, e2m1 table, e4m3 encode of a fixed ramp

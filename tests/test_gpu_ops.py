@@ -269,6 +269,28 @@ def test_act_quant_bit_exact_vs_oracle(hip, oracle, dtype):
     assert np.array_equal(np.exp2(sbytes.astype(np.float64) - 127), so.astype(np.float64))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_act_quant_two_terms_bit_exact_vs_oracle(hip, oracle, dtype):
+    """Both terms of the two-term quantiser: codes and scales equal the oracle's, which is the reference's
+    quantiser applied to x and then to what it leaves over."""
+    rng = np.random.default_rng(6)
+    x = (rng.normal(0, 1, (48, 512)) * np.repeat(10.0 ** rng.uniform(-4, 4, (48, 16)), 32, axis=1)).astype(np.float32)
+    x[2, 64:96] = 0.0
+    x[4, 0:32] = np.linspace(7.3 / 512, 8.1 / 512, 32)
+    x[4, 0] = 448.0
+    x[6, 32:64] = 2.0 ** -120          # scales at the smallest normal
+    xt = torch.from_numpy(x).to(dtype)
+    xr = xt.to(torch.float32).numpy()
+    q1, s1, q2, s2 = (host(hip, t).ravel() for t in hip.act_quant_fp8_x2(xt.to(hip.device)))
+    o1, t1, o2, t2 = oracle.act_quant_fp8_x2(xr)
+    assert np.array_equal(q1, o1) and np.array_equal(q2, o2)
+    assert np.array_equal(np.exp2(s1.astype(np.float64) - 127), t1.astype(np.float64))
+    assert np.array_equal(np.exp2(s2.astype(np.float64) - 127), t2.astype(np.float64))
+    # the first term is the one-term quantiser's output
+    q, s = hip.act_quant_fp8(xt.to(hip.device))
+    assert np.array_equal(host(hip, q).ravel(), q1) and np.array_equal(host(hip, s).ravel(), s1)
+
+
 def test_pack_is_a_pure_permutation(hip, oracle):
     """dequant(packed) == dequant(checkpoint layout) for every matrix of several experts, bit for bit."""
     cfg = synth.MoeConfig(4, 256, 3, 2, 128, 256, 1, 1)

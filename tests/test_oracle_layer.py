@@ -84,24 +84,86 @@ def test_layer_token_subset_equals_full(oracle):
     assert np.array_equal(sub["ids"], full["ids"])
 
 
-def test_layer_fp8_activation_mode_is_quantise_then_f32(oracle):
-    """act_mode 1 == act_mode 0 on activations that are already fixed points of the e4m3/32 quantiser at
-    both quantisation points is hard to arrange; instead check the definition on the first GEMM: feeding the
-    dequantised x to the f32 layer reproduces everything up to the second quantisation (down input)."""
-    inp = synth.make_inputs(synth.CONFIGS["c0"], seed=2)
-    q, s = oracle.act_quant_fp8(inp.x, 32, True)
-    xdq = (np.array([oracle.e4m3_decode(int(b)) for b in q], np.float32) * np.repeat(s, 32)).reshape(inp.x.shape)
-    a = oracle.moe_ffn_mxfp4(inp, act_mode=1)
-    # routing always sees the unquantised x
-    b = oracle.moe_ffn_mxfp4(inp, act_mode=0)
-    assert np.array_equal(a["ids"], b["ids"]) and np.array_equal(a["probs"], b["probs"])
-    err = refmath.max_abs_rel(a["out"], b["out"])
-    assert 1e-4 < err < 6e-2, err      # e4m3 has 3 mantissa bits: a few percent, not zero
-    # quantising the dequantised x again reproduces the same values (the scale may drop a binade when the
-    # block maximum rounded down onto a power of two; the represented numbers do not move)
-    q2, s2 = oracle.act_quant_fp8(xdq, 32, True)
-    xdq2 = (np.array([oracle.e4m3_decode(int(b)) for b in q2], np.float32) * np.repeat(s2, 32)).reshape(inp.x.shape)
-    assert np.array_equal(xdq2, xdq)
+def _layer_cases():
+    c0 = synth.CONFIGS["c0"]
+    ragged = synth.MoeConfig(13, 384, 8, 3, 256, 128, 4, 2)      # blocks that do not line up with anything
+    return [(c0, 0), (c0, 2), (ragged, 5)]
+
+
+@pytest.mark.parametrize("cfg,seed", _layer_cases())
+def test_layer_quantised_activation_modes_match_an_independent_statement(oracle, cfg, seed):
+    """act_mode 1 / 2 of the oracle against a NumPy statement that shares nothing with it: float64 GEMMs,
+    torch.float8_e4m3fn casts with the reference's power-of-two block-32 scale (quant.rs:190-214), quantisation of x
+    in front of gate/up and of the SwiGLU output in front of down, where the reference's device chain quantises
+    (kernels.rs:97-108,586-598).  Agreement to 1e-6 of the output's range; and statements that quantise differently
+    (block 128, an unrounded scale, x only, the SwiGLU output only, one term where two are meant) are told apart."""
+    inp = synth.make_inputs(cfg, seed=seed)
+    # e4m3 is a floating-point format: under a power-of-two scale a value keeps its three mantissa bits whatever
+    # block its scale was taken from, until it falls below the format's range (2^-15 of the block maximum).  So the
+    # block size only shows when neighbouring blocks differ by more than that, and then only if the small blocks
+    # still matter to the result.  Every other block of 32 is therefore made 2^-16 times smaller, in x and (through
+    # the up projection's scales) in the SwiGLU output, and the weights that multiply those blocks 2^16 times
+    # larger: the f32 result is of the same kind as before, a quantiser over 32 values still sees each block at its
+    # own magnitude, and one over 128 flushes half of the blocks.
+    H, I, Is = cfg.hidden, cfg.inter, cfg.shared_inter
+    odd = lambda nblk: (np.arange(nblk) % 2) * 16
+    inp.x = (inp.x * np.repeat(2.0 ** -odd(H // 32), 32)).astype(np.float32)
+    for name in ("gate_s", "up_s", "sh_gate_s", "sh_up_s"):          # [.., rows, H/32]: columns of the small x blocks
+        setattr(inp, name, (getattr(inp, name) + odd(H // 32)[None, None, :]).astype(np.uint8))
+    for name, rows in (("up_s", I), ("sh_up_s", Is)):                # rows of the up projection -> small act blocks
+        setattr(inp, name, (getattr(inp, name) - np.repeat(odd(rows // 32), 32)[None, :, None]).astype(np.uint8))
+    for name, rows in (("down_s", I), ("sh_down_s", Is)):            # [.., H, I/32]: columns of the small act blocks
+        setattr(inp, name, (getattr(inp, name) + odd(rows // 32)[None, None, :]).astype(np.uint8))
+    f32 = oracle.moe_ffn_mxfp4(inp, act_mode=0)
+    ids, probs = f32["ids"].astype(int), f32["probs"].astype(np.float64)
+    q1, q2 = refmath.qdq_e4m3, refmath.qdq_e4m3_x2
+    q2_128 = lambda a: q1(a, block=128) + q1(np.asarray(a, np.float32) - q1(a, block=128).astype(np.float32), block=128)
+    got1 = oracle.moe_ffn_mxfp4(inp, act_mode=1)
+    got2 = oracle.moe_ffn_mxfp4(inp, act_mode=2)
+    for got in (got1, got2):       # routing sees the unquantised x
+        assert np.array_equal(got["ids"], f32["ids"]) and np.array_equal(got["probs"], f32["probs"])
+    ref1 = refmath.moe_layer(inp, ids, probs, quant_x=q1, quant_act=q1)[0]
+    ref2 = refmath.moe_layer(inp, ids, probs, quant_x=q2, quant_act=q2)[0]
+    assert refmath.max_abs_rel(got1["out"], ref1) < 1e-6
+    # the second term quantises a residual sixteen times smaller than the value, so the last-bit differences between
+    # this float64 SwiGLU and the oracle's f32 one move a rounding decision now and then: one e4m3 step of a
+    # residual, 2^-8 of one activation
+    assert refmath.max_abs_rel(got2["out"], ref2) < 1e-5
+    wrong = {
+        "block 128": dict(quant_x=lambda a: refmath.qdq_e4m3(a, block=128), quant_act=lambda a: refmath.qdq_e4m3(a, block=128)),
+        "scale not a power of two": dict(quant_x=lambda a: refmath.qdq_e4m3(a, pow2_scale=False),
+                                         quant_act=lambda a: refmath.qdq_e4m3(a, pow2_scale=False)),
+        "x only": dict(quant_x=q1, quant_act=None),
+        "SwiGLU output only": dict(quant_x=None, quant_act=q1),
+        "two terms": dict(quant_x=q2, quant_act=q2),
+    }
+    for name, kw in wrong.items():
+        assert refmath.max_abs_rel(got1["out"], refmath.moe_layer(inp, ids, probs, **kw)[0]) > 1e-3, name
+    for name, kw in {"one term": dict(quant_x=q1, quant_act=q1), "second term on x only": dict(quant_x=q2, quant_act=q1),
+                     "second term on the SwiGLU output only": dict(quant_x=q1, quant_act=q2),
+                     "block 128": dict(quant_x=q2_128, quant_act=q2_128), "no quantisation": dict()}.items():
+        assert refmath.max_abs_rel(got2["out"], refmath.moe_layer(inp, ids, probs, **kw)[0]) > 2e-4, name
+    # distances to the f32 golden (CpuBackend proper): one e4m3 term is a few percent, two are bf16-class
+    d1, d2 = refmath.max_abs_rel(got1["out"], f32["out"]), refmath.max_abs_rel(got2["out"], f32["out"])
+    assert 5e-3 < d1 < 8e-2 and d2 < 5e-3 and d2 < d1 / 8, (d1, d2)
+
+
+def test_two_term_quantiser_is_the_quantiser_twice(oracle):
+    """fo_act_quant_fp8_x2 = act_quant_fp8 of x, then of x - dq1 (f32), bit for bit; and the two terms together
+    represent x far better than one (residual below 2^-7 of the block maximum)."""
+    rng = np.random.default_rng(4)
+    x = np.concatenate([rng.normal(0, 1, 4096), rng.normal(0, 1e-3, 512), rng.uniform(-500, 500, 512),
+                        np.zeros(64), [448.0, -448.0, 7.6 / 512, 1e-30] * 8]).astype(np.float32)
+    q1, s1, q2, s2 = oracle.act_quant_fp8_x2(x)
+    a1, b1 = oracle.act_quant_fp8(x, 32, True)
+    dq1 = np.array([oracle.e4m3_decode(int(b)) for b in a1], np.float32) * np.repeat(b1, 32)
+    a2, b2 = oracle.act_quant_fp8(x - dq1, 32, True)
+    assert np.array_equal(q1, a1) and np.array_equal(s1, b1) and np.array_equal(q2, a2) and np.array_equal(s2, b2)
+    dq2 = np.array([oracle.e4m3_decode(int(b)) for b in q2], np.float32) * np.repeat(s2, 32)
+    assert np.allclose(refmath.qdq_e4m3_x2(x), (dq1 + dq2).astype(np.float64), rtol=0, atol=0)
+    amax = np.repeat(np.abs(x.reshape(-1, 32)).max(axis=1), 32)
+    assert (np.abs(x - (dq1 + dq2)) <= amax * 2.0 ** -7 + 1e-37).all()
+    assert np.abs(x - dq1).max() >= 16 * np.abs(x - (dq1 + dq2)).max()   # four more bits at the least
 
 
 def test_golden_c0(oracle):
@@ -114,6 +176,7 @@ def test_golden_c0(oracle):
     assert np.array_equal(got["logits"], g["logits"])
     assert np.array_equal(got["out"], g["out_f32"])
     assert np.array_equal(oracle.moe_ffn_mxfp4(inp, act_mode=1)["out"], g["out_fp8act"])
+    assert np.array_equal(oracle.moe_ffn_mxfp4(inp, act_mode=2)["out"], g["out_fp8x2"])
     t = oracle.moe_permute(g["ids"], inp.cfg.n_experts)
     for k in ("counts", "starts", "perm_map", "gather_src"):
         assert np.array_equal(t[k], g[k])

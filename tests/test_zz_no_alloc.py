@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from ferrite_amd import synth
-from ferrite_amd.backend import (DT_F32, ERR_WORKSPACE, MODE_F32_CHECK, MODE_MFMA_FP8, STATIC_WORKSPACE_BYTES,
+from ferrite_amd.backend import (MODE_F32_CHECK, MODE_MFMA_FP8, MODE_MFMA_FP8_X2, STATIC_WORKSPACE_BYTES,
                                  FerriteError)
 
 pytestmark = pytest.mark.gpu
@@ -29,7 +29,7 @@ def both(hip, layer, x_np, mode, bf16=False):
     return got.cpu().numpy(), want.cpu().numpy()
 
 
-@pytest.mark.parametrize("mode", [MODE_MFMA_FP8, MODE_F32_CHECK])
+@pytest.mark.parametrize("mode", [MODE_MFMA_FP8, MODE_MFMA_FP8_X2, MODE_F32_CHECK])
 def test_static_workspace_equals_caller_workspace_twice_second_smaller(hip, mode):
     cfg = synth.MoeConfig(40, 256, 8, 3, 256, 128, 4, 2)
     inp = synth.make_inputs(cfg, seed=3)
@@ -61,10 +61,11 @@ def test_static_workspace_decode_shape(hip):
     """The decode benchmark shape (32 tokens, H 4096, 128 experts, top-8, I 1536) fits the built-in workspace."""
     inp = synth.make_inputs(synth.CONFIGS["c1"], seed=0)
     layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
-    got, want = both(hip, layer, inp.x, MODE_MFMA_FP8, bf16=True)
-    assert np.isfinite(want).all() and np.array_equal(got, want)
-    got, want = both(hip, layer, inp.x[:5], MODE_MFMA_FP8, bf16=True)
-    assert np.array_equal(got, want)
+    for mode in (MODE_MFMA_FP8_X2, MODE_MFMA_FP8):
+        got, want = both(hip, layer, inp.x, mode, bf16=True)
+        assert np.isfinite(want).all() and np.array_equal(got, want)
+        got, want = both(hip, layer, inp.x[:5], mode, bf16=True)
+        assert np.array_equal(got, want)
 
 
 def test_static_workspace_under_graph_capture(hip):
