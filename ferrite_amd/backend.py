@@ -603,36 +603,45 @@ class HipBackend:
         return layer._ws[key]
 
     def moe_block_mxfp4(self, layer: MoeLayer, li: torch.Tensor, norm_w: torch.Tensor, eps: float,
-                        residual: torch.Tensor, post: torch.Tensor, comb: torch.Tensor, out: torch.Tensor,
-                        mode: int = MODE_MFMA_FP8):
+                        residual: Optional[torch.Tensor], post: Optional[torch.Tensor], comb: Optional[torch.Tensor],
+                        out: torch.Tensor, mode: int = MODE_MFMA_FP8, workspace: Optional[torch.Tensor] = None):
         """The FFN half of a decoder layer (exec/lib.rs:487-492): rmsnorm -> MoE FFN -> hc_post, one call.
-        li [n,H] f32, residual/out [n,nh,H] f32, post [n,nh], comb [n,nh,nh]."""
+        li [n,H] f32, residual/out [n,nh,H] f32, post [n,nh], comb [n,nh,nh].  residual None: rmsnorm -> MoE FFN
+        only, out [n,H]."""
         self.recorder.record("moe_block_mxfp4")
         self._leave()
         cfg = layer.cfg
         if li.dim() != 2 or li.shape[1] != cfg.hidden:
             raise ShapeMismatch(f"li {tuple(li.shape)} vs hidden {cfg.hidden}")
         n = li.shape[0]
-        nh = residual.shape[1] if residual.dim() == 3 else -1
-        if (tuple(residual.shape) != (n, nh, cfg.hidden) or tuple(out.shape) != (n, nh, cfg.hidden)
-                or tuple(post.shape) != (n, nh) or tuple(comb.shape) != (n, nh, nh) or norm_w.numel() != cfg.hidden):
-            raise ShapeMismatch("moe_block shape mismatch")
-        for t, nm in ((li, "li"), (norm_w, "norm_w"), (residual, "residual"), (post, "post"), (comb, "comb"),
-                      (out, "out")):
+        tensors = [(li, "li"), (norm_w, "norm_w"), (out, "out")]
+        if residual is None:
+            nh = 0
+            if tuple(out.shape) != (n, cfg.hidden) or norm_w.numel() != cfg.hidden:
+                raise ShapeMismatch("moe_block shape mismatch")
+        else:
+            nh = residual.shape[1] if residual.dim() == 3 else -1
+            if (tuple(residual.shape) != (n, nh, cfg.hidden) or tuple(out.shape) != (n, nh, cfg.hidden)
+                    or tuple(post.shape) != (n, nh) or tuple(comb.shape) != (n, nh, nh) or norm_w.numel() != cfg.hidden):
+                raise ShapeMismatch("moe_block shape mismatch")
+            tensors += [(residual, "residual"), (post, "post"), (comb, "comb")]
+        for t, nm in tensors:
             self._dev(t, torch.float32, nm)
         if mode != MODE_F32_CHECK and layer.packed is None:
             raise InvalidArg("layer has no packed weights")
-        ws = self.block_workspace(layer, n, mode)
-        blk = MoeBlockArgs(norm_w.data_ptr(), eps, residual.data_ptr(), post.data_ptr(), comb.data_ptr(), nh)
+        ws = workspace if workspace is not None else self.block_workspace(layer, n, mode)
+        ptr = lambda t: None if t is None else t.data_ptr()
+        blk = MoeBlockArgs(norm_w.data_ptr(), eps, ptr(residual), ptr(post), ptr(comb), nh)
         self._enter()
         self._ck(self.lib.ferrite_moe_block_mxfp4(C.byref(layer.shape), C.byref(layer.weights),
                                                   None if layer.packed is None else layer.packed.data_ptr(),
                                                   li.data_ptr(), C.byref(blk), n, out.data_ptr(), mode, ws.data_ptr(),
                                                   ws.numel(), self._st()), "moe_block_mxfp4")
 
-    def workspace_view(self, layer: MoeLayer, n: int, mode: int) -> Dict[str, torch.Tensor]:
+    def workspace_view(self, layer: MoeLayer, n: int, mode: int,
+                       workspace: Optional[torch.Tensor] = None) -> Dict[str, torch.Tensor]:
         """Typed views of the intermediates the last layer call left in its workspace."""
-        ws = self.workspace(layer, n, mode)
+        ws = workspace if workspace is not None else self.workspace(layer, n, mode)
         v = WorkspaceView()
         self._ck(self.lib.ferrite_moe_layer_workspace_view(C.byref(layer.shape), n, mode, ws.data_ptr(), C.byref(v)),
                  "workspace_view")
@@ -646,7 +655,7 @@ class HipBackend:
             return ws[off:off + count * size].view(dtype)
 
         E, k = cfg.n_experts, cfg.topk
-        y_bf16 = (mode == MODE_MFMA_FP8 and self.unit_rows(layer, n, mode) == 128
+        y_bf16 = (mode != MODE_F32_CHECK and self.unit_rows(layer, n, mode) == 128
                   and not self._overrides[OVERRIDE_Y_F32])
         y_dtype = torch.bfloat16 if y_bf16 else torch.float32
         return dict(logits=view(v.logits, n * E, torch.float32).view(n, E),

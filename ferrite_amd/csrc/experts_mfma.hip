@@ -100,20 +100,41 @@ __global__ __launch_bounds__(256) void pack_scales_kernel(PackSrc s, int n_exper
 }
 
 // ---- the streaming core ---------------------------------------------------------------------------
-// One wave, one item: for every k step, 4 A tiles from global memory (16 B per lane each), B from LDS, 4 MFMAs.
-// bq: [KT][2][64] uint4 (the unit's activations in operand order), bsc: [KT4][64] u32 (their scales).
-template <int Q>
-__device__ __forceinline__ void mfma_step(const u4v (&a)[4], const u4v& sc, const u4v* bq, uint32_t bscale,
-                                          int kt, int lane, v4f (&acc)[4]) {
-    const u4v b0 = bq[(kt * 2 + 0) * 64 + lane];
-    const u4v b1 = bq[(kt * 2 + 1) * 64 + lane];
-    const v8i bv = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+// One wave, one item: for every k step, 4 A tiles from global memory (16 B per lane each), B from LDS, 4 MFMAs
+// (8 with two-term activations: the same weight registers against each term's plane).
+// The B operand in LDS covers one window of k steps: bq [window k steps][2][64] uint4 (the unit's activations in
+// operand order), bsc [window groups of 4 k steps][64] u32 (their scales); bq2 / bsc2 the second term's plane.
+struct BWindow {
+    const u4v* bq;
+    const u4v* bq2;
+    const uint32_t* bsc;
+    const uint32_t* bsc2;
+};
+
+template <int Q, bool kX2>
+__device__ __forceinline__ void mfma_step(const u4v (&a)[4], const u4v& sc, const BWindow& b, uint32_t bs, uint32_t bs2,
+                                          int ktw, int lane, v4f (&acc)[4]) {
     const uint32_t scs[4] = {sc[0], sc[1], sc[2], sc[3]};
+    {
+        const u4v b0 = b.bq[(ktw * 2 + 0) * 64 + lane];
+        const u4v b1 = b.bq[(ktw * 2 + 1) * 64 + lane];
+        const v8i bv = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        const v8i av = {(int)a[t][0], (int)a[t][1], (int)a[t][2], (int)a[t][3], 0, 0, 0, 0};
-        acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[t], 4 /*A e2m1*/, 0 /*B e4m3*/, Q,
-                                                                  (int)scs[t], Q, (int)bscale);
+        for (int t = 0; t < 4; ++t) {
+            const v8i av = {(int)a[t][0], (int)a[t][1], (int)a[t][2], (int)a[t][3], 0, 0, 0, 0};
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[t], 4 /*A e2m1*/, 0 /*B e4m3*/, Q,
+                                                                      (int)scs[t], Q, (int)bs);
+        }
+    }
+    if constexpr (kX2) {
+        const u4v b0 = b.bq2[(ktw * 2 + 0) * 64 + lane];
+        const u4v b1 = b.bq2[(ktw * 2 + 1) * 64 + lane];
+        const v8i bv = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const v8i av = {(int)a[t][0], (int)a[t][1], (int)a[t][2], (int)a[t][3], 0, 0, 0, 0};
+            acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[t], 4, 0, Q, (int)scs[t], Q, (int)bs2);
+        }
     }
 }
 
@@ -146,81 +167,158 @@ __device__ __forceinline__ void stream_load_group(StreamRegs& r, const u4v* __re
     }
 }
 
-// The item's group 0 must already be in flight in buffer 0 (stream_load_group(..., 0, 0)): callers issue it
-// before they fill LDS, so the first weights travel while the activations are staged.
-template <bool kKeep>
+template <bool kX2, int BUF>
+__device__ __forceinline__ void stream_group(const StreamRegs& r, const BWindow& b, int KT, int g4, int g4w, int lane,
+                                             v4f (&acc)[4]) {
+    const uint32_t bs = b.bsc[g4w * 64 + lane];
+    uint32_t bs2 = 0;
+    if constexpr (kX2) bs2 = b.bsc2[g4w * 64 + lane];
+    const int kt = g4 * 4, ktw = g4w * 4;
+    mfma_step<0, kX2>(r.a[BUF][0], r.sc[BUF], b, bs, bs2, ktw, lane, acc);
+    if (kt + 1 < KT) mfma_step<1, kX2>(r.a[BUF][1], r.sc[BUF], b, bs, bs2, ktw + 1, lane, acc);
+    if (kt + 2 < KT) mfma_step<2, kX2>(r.a[BUF][2], r.sc[BUF], b, bs, bs2, ktw + 2, lane, acc);
+    if (kt + 3 < KT) mfma_step<3, kX2>(r.a[BUF][3], r.sc[BUF], b, bs, bs2, ktw + 3, lane, acc);
+}
+
+// Groups [g_lo, g_hi) of the item against the window in LDS (whose first group is g_lo).  Group g_lo must already
+// be in flight in buffer 0: callers issue group 0 before they fill LDS, so the first weights travel while the
+// activations are staged, and every window but the last holds an even number of groups, so a window ends with the
+// next one's first group in flight in buffer 0 again.  Loads run ahead to the item's last group (KT4) whatever the
+// window.
+template <bool kKeep, bool kX2>
 __device__ __forceinline__ void stream_item(StreamRegs& r, const u4v* __restrict__ wp, const u4v* __restrict__ sp,
-                                            int KT, const u4v* bq, const uint32_t* bsc, int lane, v4f (&acc)[4]) {
+                                            int KT, int g_lo, int g_hi, const BWindow& b, int lane, v4f (&acc)[4]) {
     const int KT4 = (KT + 3) >> 2;
-    for (int g4 = 0; g4 < KT4; g4 += 2) {
+    for (int g4 = g_lo; g4 < g_hi; g4 += 2) {
         if (g4 + 1 < KT4) stream_load_group<kKeep>(r, wp, sp, KT, lane, g4 + 1, 1);
-        {
-            const uint32_t bs = bsc[g4 * 64 + lane];
-            const int kt = g4 * 4;
-            mfma_step<0>(r.a[0][0], r.sc[0], bq, bs, kt, lane, acc);
-            if (kt + 1 < KT) mfma_step<1>(r.a[0][1], r.sc[0], bq, bs, kt + 1, lane, acc);
-            if (kt + 2 < KT) mfma_step<2>(r.a[0][2], r.sc[0], bq, bs, kt + 2, lane, acc);
-            if (kt + 3 < KT) mfma_step<3>(r.a[0][3], r.sc[0], bq, bs, kt + 3, lane, acc);
-        }
-        if (g4 + 1 < KT4) {
+        stream_group<kX2, 0>(r, b, KT, g4, g4 - g_lo, lane, acc);
+        if (g4 + 1 < g_hi) {
             if (g4 + 2 < KT4) stream_load_group<kKeep>(r, wp, sp, KT, lane, g4 + 2, 0);
-            const uint32_t bs = bsc[(g4 + 1) * 64 + lane];
-            const int kt = (g4 + 1) * 4;
-            mfma_step<0>(r.a[1][0], r.sc[1], bq, bs, kt, lane, acc);
-            if (kt + 1 < KT) mfma_step<1>(r.a[1][1], r.sc[1], bq, bs, kt + 1, lane, acc);
-            if (kt + 2 < KT) mfma_step<2>(r.a[1][2], r.sc[1], bq, bs, kt + 2, lane, acc);
-            if (kt + 3 < KT) mfma_step<3>(r.a[1][3], r.sc[1], bq, bs, kt + 3, lane, acc);
+            stream_group<kX2, 1>(r, b, KT, g4 + 1, g4 + 1 - g_lo, lane, acc);
         }
     }
 }
 
-// Copies the e4m3 rows of a unit into LDS in B-operand order and builds the packed scale words.
-// row_src(r) gives the source row of unit row r (or -1).  Source rows are `pitch` bytes apart, of which the first K
-// are read; scale rows are in operand order (scale_pos), `spitch` bytes apart.
-// kX2: the activations are two-term (value ~ term 1 + term 2, each e4m3 per 32 with its own scales, in two planes
-// of the same shape).  A unit then has at most 8 rows, and the 16 operand columns hold term 1 of row c in column c
-// and term 2 of row c in column c + 8: one instruction multiplies both terms by the weights, and the two partial
-// results of a row meet in the epilogue (lanes c and c ^ 8).  No more instructions and no more LDS than one term
-// for 16 rows.
+// Where a unit's activations live in LDS while its weights stream past: the whole reduction length (K x 16 bytes
+// per term), or windows of kWindowKt k steps.  Two-term activations of a long reduction need 2 x 16 x K bytes
+// (K 4096: 128 KiB), which leaves no room for a second block on the CU; staged in windows of 2048 k they take
+// 64 KiB + scales per block whatever K is.  Between two windows the block's waves meet at a barrier, refill LDS
+// and meet again.  A window is a multiple of two groups (see stream_item).
+constexpr int kWindowKt = 16;
+
+// WIN: k steps per window, 0 = the whole reduction resident.
+template <int WIN>
+__host__ __device__ __forceinline__ int window_kt(int KT) { return WIN > 0 && KT > WIN ? WIN : KT; }
+template <bool kX2, int WIN>
+static inline size_t b_lds_bytes(int KT) {
+    const int w = window_kt<WIN>(KT);
+    return (size_t)(kX2 ? 2 : 1) * ((size_t)w * 2048 + (size_t)((w + 3) / 4) * 256);
+}
+
+// The planes of a window of w k steps at `lds`.
+template <bool kX2>
+struct BPlanes {
+    u4v *bq, *bq2;
+    uint32_t *bsc, *bsc2;
+    __device__ __forceinline__ BPlanes(unsigned char* lds, int w) {
+        const size_t codes = (size_t)w * 2048, scales = (size_t)((w + 3) / 4) * 256;
+        bq = reinterpret_cast<u4v*>(lds);
+        bq2 = kX2 ? reinterpret_cast<u4v*>(lds + codes) : nullptr;
+        bsc = reinterpret_cast<uint32_t*>(lds + (kX2 ? 2 : 1) * codes);
+        bsc2 = kX2 ? reinterpret_cast<uint32_t*>(lds + 2 * codes + scales) : nullptr;
+    }
+    __device__ __forceinline__ BWindow window() const { return BWindow{bq, bq2, bsc, bsc2}; }
+};
+
+// One 16-byte chunk / one scale word of a window: where it comes from and which slot of the B operand it fills.
+// row_src(r) gives the source row of unit row r (or -1).  Source rows are `pitch` bytes apart; scale rows are in
+// operand order (scale_pos), `spitch` bytes apart.
+template <bool kX2>
+struct BSource {
+    ActPlanes src;
+    size_t pitch;
+    int spitch, nrows;
+};
+
 template <bool kX2, typename RowFn>
-__device__ __forceinline__ void fill_b_operand(const uint8_t* __restrict__ q, const uint8_t* __restrict__ qs,
-                                               const uint8_t* __restrict__ q2, const uint8_t* __restrict__ qs2, int K,
-                                               size_t pitch, int spitch, int nrows, RowFn row_src, u4v* bq,
-                                               uint32_t* bsc) {
-    const int chunks = K / 16;
-    const int ncols = kX2 ? 16 : nrows;
-    for (int idx = threadIdx.x; idx < ncols * chunks; idx += blockDim.x) {
-        const int c = idx / chunks, j = idx % chunks;
-        const int ur = kX2 ? (c & 7) : c;
-        if (kX2 && ur >= nrows) continue;
-        const int r = row_src(ur);
-        const uint8_t* plane = (kX2 && c >= 8) ? q2 : q;
-        u4v v = {0u, 0u, 0u, 0u};
-        if (r >= 0) v = *reinterpret_cast<const u4v*>(plane + (size_t)r * pitch + (size_t)j * 16);
-        const int k = j * 16, kt = k >> 7, within = k & 127;
-        const int half = within >> 6, g = (within & 63) >> 4;
-        bq[(kt * 2 + half) * 64 + g * 16 + c] = v;
+__device__ __forceinline__ int b_chunk(const BSource<kX2>& s, RowFn row_src, int kt0, int wkt, int idx, u4v& v) {
+    const int chunks = wkt * 8;   // 16-byte chunks per row and plane in the window
+    const int p = idx / (s.nrows * chunks), rem = idx - p * (s.nrows * chunks);
+    const int c = rem / chunks, j = rem % chunks;
+    const int r = row_src(c);
+    const uint8_t* plane = p ? s.src.q2 : s.src.q;
+    v = (u4v){0u, 0u, 0u, 0u};
+    if (r >= 0) v = *reinterpret_cast<const u4v*>(plane + (size_t)r * s.pitch + (size_t)kt0 * 128 + (size_t)j * 16);
+    const int ktw = j >> 3, within = (j & 7) * 16;
+    const int half = within >> 6, g = (within & 63) >> 4;
+    return (p << 30) | ((ktw * 2 + half) * 64 + g * 16 + c);
+}
+
+template <bool kX2, typename RowFn>
+__device__ __forceinline__ int b_scale_word(const BSource<kX2>& s, RowFn row_src, int kt0, int wkt, int idx, uint32_t& v) {
+    const int wg = (wkt + 3) / 4;
+    const int p = idx / (wg * 64), rem = idx - p * (wg * 64);
+    const int k4 = rem >> 6, l = rem & 63, c = l & 15, g = l >> 4;
+    v = 0x7f7f7f7fu;
+    if (c < s.nrows) {
+        const int r = row_src(c);
+        const uint8_t* plane = p ? s.src.s2 : s.src.s;
+        if (r >= 0) v = *reinterpret_cast<const uint32_t*>(plane + (size_t)r * s.spitch + (kt0 / 4 + k4) * 16 + g * 4);
     }
-    const int KT = K / 128, KT4 = (KT + 3) / 4;
-    for (int idx = threadIdx.x; idx < KT4 * 64; idx += blockDim.x) {
-        const int k4 = idx >> 6, l = idx & 63, c = l & 15, g = l >> 4;
-        const int ur = kX2 ? (c & 7) : c;
-        uint32_t v = 0x7f7f7f7fu;
-        if (ur < nrows) {
-            const int r = row_src(ur);
-            const uint8_t* plane = (kX2 && c >= 8) ? qs2 : qs;
-            if (r >= 0) v = *reinterpret_cast<const uint32_t*>(plane + (size_t)r * spitch + k4 * 16 + g * 4);
-        }
-        bsc[idx] = v;
+    return (p << 30) | rem;
+}
+
+// Copies k steps [kt0, kt0 + wkt) of the unit's rows into LDS in B-operand order and builds the packed scale words
+// (any window length; loads and stores alternate).
+template <bool kX2, typename RowFn>
+__device__ __forceinline__ void fill_b_window(const BSource<kX2>& s, RowFn row_src, int kt0, int wkt,
+                                              const BPlanes<kX2>& d) {
+    constexpr int NP = kX2 ? 2 : 1;
+    const int total = NP * s.nrows * wkt * 8;
+    for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
+        u4v v;
+        const int slot = b_chunk<kX2>(s, row_src, kt0, wkt, idx, v);
+        ((slot >> 30) ? d.bq2 : d.bq)[slot & 0x3fffffff] = v;
+    }
+    const int wg = (wkt + 3) / 4;
+    for (int idx = threadIdx.x; idx < NP * wg * 64; idx += blockDim.x) {
+        uint32_t v;
+        const int slot = b_scale_word<kX2>(s, row_src, kt0, wkt, idx, v);
+        ((slot >> 30) ? d.bsc2 : d.bsc)[slot & 0x3fffffff] = v;
     }
 }
 
-// Two-term activations: lanes c and c ^ 8 of a 16-lane row hold the partial results of the same unit row.
-__device__ __forceinline__ void join_terms(v4f (&acc)[4]) {
+// The reduction of `rounds` items per wave against one unit's activation rows.  item(round, wp, sp) gives the
+// round's weight stream of this wave (false: no item, the wave only keeps the barriers company); the first round's
+// group 0 must already be in flight in buffer 0.  done(round, acc) receives the finished accumulators.  Every wave of the block makes the same calls: the barriers inside are block-wide.
+template <bool kKeep, bool kX2, int WIN, typename RowFn, typename ItemFn, typename DoneFn>
+__device__ __forceinline__ void run_unit(const BSource<kX2>& s, RowFn row_src, int KT, int rounds, ItemFn item, DoneFn done,
+                                         StreamRegs& regs, unsigned char* lds, int lane) {
+    const int WKT = window_kt<WIN>(KT), nw = (KT + WKT - 1) / WKT;
+    const BPlanes<kX2> d(lds, WKT);
+    const BWindow win = d.window();
+    bool filled = false;
+#pragma unroll 1
+    for (int r = 0; r < rounds; ++r) {
+        const u4v *wp, *sp;
+        const bool live = item(r, wp, sp);
+        if (r > 0 && live) stream_load_group<kKeep>(regs, wp, sp, KT, lane, 0, 0);
+        v4f acc[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) acc[t][v] += __shfl_xor(acc[t][v], 8, 64);
+        for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+        for (int w = 0; w < nw; ++w) {
+            const int kt0 = w * WKT, wkt = min(WKT, KT - kt0);
+            if (nw > 1 || !filled) {
+                if (filled) __syncthreads();   // every wave is done with the window that is in LDS
+                fill_b_window<kX2>(s, row_src, kt0, wkt, d);
+                __syncthreads();
+                filled = true;
+            }
+            if (live) stream_item<kKeep, kX2>(regs, wp, sp, KT, kt0 / 4, (kt0 + wkt + 3) / 4, win, lane, acc);
+        }
+        if (live) done(r, acc);
+    }
 }
 
 struct MfmaArgs {
@@ -265,10 +363,10 @@ __device__ __forceinline__ bool unit_block_work(const MfmaArgs& a, int groups, i
     return true;
 }
 
-// gate/up GEMM + clamped SwiGLU + e4m3-per-32 quantisation of the result.
+// gate/up GEMM + clamped SwiGLU + e4m3-per-32 quantisation of the result (one or two terms).
 // grid: unit_block_work over groups = ceil(items / WAVES) item groups; wave w of item group ig owns item
 // ig*WAVES + w of the unit's expert.
-template <int WAVES, bool kKeep, bool kX2>
+template <int WAVES, bool kKeep, bool kX2, int WIN>
 __device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& xin,
                                              const int32_t* __restrict__ gather_src, const ActPlanes& act,
                                              unsigned char* lds_raw) {
@@ -279,8 +377,6 @@ __device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, c
     const int items = inter / 32;
     if (ig * WAVES >= items) return;
     const int H = a.hidden, KT = H / 128, KT4 = (KT + 3) / 4;
-    u4v* bq = reinterpret_cast<u4v*>(lds_raw);
-    uint32_t* bsc = reinterpret_cast<uint32_t*>(lds_raw + (size_t)H * 16);
     const int nk = a.n * a.topk, topk = a.topk;
     auto row_src = [&](int c) -> int {
         int g = row0 + c;
@@ -293,75 +389,79 @@ __device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, c
     const bool live = item < items;
     const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
     const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
-    const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
-    const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
+    const u4v* wp0 = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
+    const u4v* sp0 = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
     StreamRegs regs;
-    if (live) stream_load_group<kKeep>(regs, wp, sp, KT, lane, 0, 0);   // weights fly while the activations are staged
-    fill_b_operand<kX2>(xin.q, xin.s, xin.q2, xin.s2, H, (size_t)H, scale_pitch(H), nrows, row_src, bq, bsc);
-    __syncthreads();
-    if (!live) return;
-    v4f acc[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-    stream_item<kKeep>(regs, wp, sp, KT, bq, bsc, lane, acc);
-    if constexpr (kX2) join_terms(acc);
-
-    // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
-    float r0[4], r1[4];
-    float amax = 0.0f;
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        r0[v] = swiglu_fast(acc[0][v], acc[2][v], a.limit);
-        r1[v] = swiglu_fast(acc[1][v], acc[3][v], a.limit);
-        amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+    if (live) {   // weights fly while the activations are staged
+        stream_load_group<kKeep>(regs, wp0, sp0, KT, lane, 0, 0);
     }
-    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-    const int c = lane & 15, g = lane >> 4;
-    const int ur = kX2 ? (c & 7) : c;
-    const uint32_t sb = block_scale_e8m0(amax);
-    const float inv = u2f((254u - sb) << 23);
-    uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
-    uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
-    uint8_t* dq = act.q;
-    uint8_t* ds = act.s;
-    uint32_t sbo = sb;
-    if constexpr (kX2) {
-        // second term: the same quantiser on what the first leaves over; lanes c >= 8 store it, lanes c < 8 the first
-        const float sc = u2f(sb << 23);
-        float amax2 = 0.0f;
+    const BSource<kX2> bsrc{xin, (size_t)H, scale_pitch(H), nrows};
+    run_unit<kKeep, kX2, WIN>(
+        bsrc, row_src, KT, 1,
+        [&](int, const u4v*& wp, const u4v*& sp) { wp = wp0; sp = sp0; return live; },
+        [&](int, v4f (&acc)[4]) {
+            // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
+            float r0[4], r1[4];
+            float amax = 0.0f;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            r0[v] = fadd(r0[v], -fmul(e4m3_decode((p0 >> (8 * v)) & 0xffu), sc));
-            r1[v] = fadd(r1[v], -fmul(e4m3_decode((p1 >> (8 * v)) & 0xffu), sc));
-            amax2 = fmaxf(amax2, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
-        }
-        amax2 = fmaxf(amax2, __shfl_xor(amax2, 16, 64));
-        amax2 = fmaxf(amax2, __shfl_xor(amax2, 32, 64));
-        const uint32_t sb2 = block_scale_e8m0(amax2);
-        const float inv2 = u2f((254u - sb2) << 23);
-        const uint32_t t0 = e4m3_encode4_hw(r0[0] * inv2, r0[1] * inv2, r0[2] * inv2, r0[3] * inv2);
-        const uint32_t t1 = e4m3_encode4_hw(r1[0] * inv2, r1[1] * inv2, r1[2] * inv2, r1[3] * inv2);
-        if (c >= 8) { p0 = t0; p1 = t1; sbo = sb2; dq = act.q2; ds = act.s2; }
-    }
-    if (ur < nrows) {
-        uint8_t* dst = dq + (size_t)(row0 + ur) * a.act_ld + (size_t)item * 32 + g * 4;
-        *reinterpret_cast<uint32_t*>(dst) = p0;
-        *reinterpret_cast<uint32_t*>(dst + 16) = p1;
-        if (g == 0) ds[(size_t)(row0 + ur) * scale_pitch(a.act_ld) + scale_pos(item)] = (uint8_t)sbo;
-    }
+            for (int v = 0; v < 4; ++v) {
+                r0[v] = swiglu_fast(acc[0][v], acc[2][v], a.limit);
+                r1[v] = swiglu_fast(acc[1][v], acc[3][v], a.limit);
+                amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+            }
+            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            const int c = lane & 15, g = lane >> 4;
+            const uint32_t sb = block_scale_e8m0(amax);
+            const float inv = u2f((254u - sb) << 23);
+            const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
+            const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
+            const size_t qoff = (size_t)(row0 + c) * a.act_ld + (size_t)item * 32 + g * 4;
+            const size_t soff = (size_t)(row0 + c) * scale_pitch(a.act_ld) + scale_pos(item);
+            if (c < nrows) {
+                *reinterpret_cast<uint32_t*>(act.q + qoff) = p0;
+                *reinterpret_cast<uint32_t*>(act.q + qoff + 16) = p1;
+                if (g == 0) act.s[soff] = (uint8_t)sb;
+            }
+            if constexpr (kX2) {
+                // second term: the same quantiser on what the first leaves over
+                const float sc = u2f(sb << 23);
+                float amax2 = 0.0f;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    r0[v] = fadd(r0[v], -fmul(e4m3_decode((p0 >> (8 * v)) & 0xffu), sc));
+                    r1[v] = fadd(r1[v], -fmul(e4m3_decode((p1 >> (8 * v)) & 0xffu), sc));
+                    amax2 = fmaxf(amax2, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+                }
+                amax2 = fmaxf(amax2, __shfl_xor(amax2, 16, 64));
+                amax2 = fmaxf(amax2, __shfl_xor(amax2, 32, 64));
+                const uint32_t sb2 = block_scale_e8m0(amax2);
+                const float inv2 = u2f((254u - sb2) << 23);
+                const uint32_t t0 = e4m3_encode4_hw(r0[0] * inv2, r0[1] * inv2, r0[2] * inv2, r0[3] * inv2);
+                const uint32_t t1 = e4m3_encode4_hw(r1[0] * inv2, r1[1] * inv2, r1[2] * inv2, r1[3] * inv2);
+                if (c < nrows) {
+                    *reinterpret_cast<uint32_t*>(act.q2 + qoff) = t0;
+                    *reinterpret_cast<uint32_t*>(act.q2 + qoff + 16) = t1;
+                    if (g == 0) act.s2[soff] = (uint8_t)sb2;
+                }
+            }
+        },
+        regs, lds_raw, lane);
 }
 
-template <int WAVES, bool kX2>
-__global__ __launch_bounds__(WAVES * 64) void gate_up_mfma_kernel(MfmaArgs a, int groups, ActPlanes xin,
-                                                                  const int32_t* __restrict__ gather_src,
-                                                                  ActPlanes act) {
+// WIN: window of the activation staging in k steps, 0 = resident (see window_kt).  One-term activations are always
+// resident; two-term ones are windowed at 2048 k with two 4-wave blocks per CU, or resident with one 8-wave block
+// per CU (the launcher chooses).
+template <int WAVES, bool kX2, int WIN>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gate_up_mfma_kernel(MfmaArgs a, int groups, ActPlanes xin,
+                                                                                      const int32_t* __restrict__ gather_src,
+                                                                                      ActPlanes act) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig, ne;
     if (!unit_block_work(a, groups, u, ig, ne)) return;
     // an expert with several units: its weights are wanted again by the blocks that follow on this XCD
-    if (ne > 1) gate_up_unit<WAVES, true, kX2>(a, u, ig, xin, gather_src, act, lds_raw);
-    else gate_up_unit<WAVES, false, kX2>(a, u, ig, xin, gather_src, act, lds_raw);
+    if (ne > 1) gate_up_unit<WAVES, true, kX2, WIN>(a, u, ig, xin, gather_src, act, lds_raw);
+    else gate_up_unit<WAVES, false, kX2, WIN>(a, u, ig, xin, gather_src, act, lds_raw);
 }
 
 // down GEMM: y[row][h] for the unit's rows.  grid: unit_block_work over groups = ceil(items / (WAVES*IPW)); item =
@@ -375,47 +475,40 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
     const int inter = shared ? a.shared_inter : a.inter;
     const int H = a.hidden, items = H / 64;
     const int KT = inter / 128, KT4 = (KT + 3) / 4;
-    u4v* bq = reinterpret_cast<u4v*>(lds_raw);
-    uint32_t* bsc = reinterpret_cast<uint32_t*>(lds_raw + (size_t)a.act_ld * 16);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int item0 = (ig * WAVES + wave) * IPW;
-    StreamRegs regs;
-    if (item0 < items) {   // the first item's weights fly while the activations are staged
-        const uint8_t* cb = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
-        const uint8_t* sb = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
-        stream_load_group<kKeep>(regs, reinterpret_cast<const u4v*>(cb) + (size_t)item0 * KT * 256,
-                          reinterpret_cast<const u4v*>(sb) + (size_t)item0 * KT4 * 64, KT, lane, 0, 0);
-    }
-    // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
-    fill_b_operand<kX2>(act.q, act.s, act.q2, act.s2, inter, (size_t)a.act_ld, scale_pitch(a.act_ld), nrows,
-                        [&](int c) { return row0 + c; }, bq, bsc);
-    __syncthreads();
     const uint8_t* cbase = shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert;
     const uint8_t* sbase = shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert;
-    const int c = lane & 15, g = lane >> 4;
-#pragma unroll 1
-    for (int ii = 0; ii < IPW; ++ii) {
-        const int item = item0 + ii;
-        if (item >= items) break;
-        const u4v* wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
-        const u4v* sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
-        if (ii > 0) stream_load_group<kKeep>(regs, wp, sp, KT, lane, 0, 0);
-        v4f acc[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-        stream_item<kKeep>(regs, wp, sp, KT, bq, bsc, lane, acc);
-        if constexpr (kX2) join_terms(acc);
-        if (c < nrows && (!kX2 || c < 8)) {
-            float* dst = y + (size_t)(row0 + c) * H + (size_t)item * 64 + g * 4;
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                *reinterpret_cast<float4*>(dst + t * 16) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-        }
+    StreamRegs regs;
+    if (item0 < items) {   // the first item's weights fly while the activations are staged
+        const u4v* wp0 = reinterpret_cast<const u4v*>(cbase) + (size_t)item0 * KT * 256;
+        const u4v* sp0 = reinterpret_cast<const u4v*>(sbase) + (size_t)item0 * KT4 * 64;
+        stream_load_group<kKeep>(regs, wp0, sp0, KT, lane, 0, 0);
     }
+    // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
+    const BSource<kX2> bsrc{act, (size_t)a.act_ld, scale_pitch(a.act_ld), nrows};
+    const int c = lane & 15, g = lane >> 4;
+    run_unit<kKeep, kX2, kX2 ? kWindowKt : 0>(
+        bsrc, [&](int col) { return row0 + col; }, KT, IPW,
+        [&](int r, const u4v*& wp, const u4v*& sp) {
+            const int item = item0 + r;
+            wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
+            sp = reinterpret_cast<const u4v*>(sbase) + (size_t)item * KT4 * 64;
+            return item < items;
+        },
+        [&](int r, v4f (&acc)[4]) {
+            if (c < nrows) {
+                float* dst = y + (size_t)(row0 + c) * H + (size_t)(item0 + r) * 64 + g * 4;
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    *reinterpret_cast<float4*>(dst + t * 16) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+            }
+        },
+        regs, lds_raw, lane);
 }
 
 template <int WAVES, int IPW, bool kX2>
-__global__ __launch_bounds__(WAVES * 64) void down_mfma_kernel(MfmaArgs a, int groups, ActPlanes act,
+__global__ __launch_bounds__(WAVES * 64, 2) void down_mfma_kernel(MfmaArgs a, int groups, ActPlanes act,
                                                                float* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig, ne;
@@ -711,6 +804,7 @@ __global__ __launch_bounds__(PF_WAVES * 64, PF_WAVES == 4 ? 2 : 1) void down_pre
 
 // ---- launchers ----------------------------------------------------------------------------------------
 constexpr int GU_WAVES = 4;
+constexpr int GU_WAVES_RESIDENT_X2 = 8;
 constexpr int DN_WAVES = 4;
 constexpr int DN_IPW = 2;
 
@@ -753,18 +847,37 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
                               k_stop, 0, a, groups, xin.q, xin.s, gather_src, act.q, act.s);
         return check_launch("gate_up_prefill");
     }
-    if (units.unit_rows_cap != (x2 ? 8 : 16)) return FERRITE_ERR_INVALID_ARG;
-    const size_t lds = (size_t)s.hidden * 16 + (size_t)((s.hidden / 128 + 3) / 4) * 256;
-    const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
-    const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
+    const int KT = s.hidden / 128;
     int rc;
     if (x2) {
-        if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true>>::ensure(lds))) return rc;
-        hipExtLaunchKernelGGL((gate_up_mfma_kernel<GU_WAVES, true>), dim3(blocks), dim3(GU_WAVES * 64), (uint32_t)lds, st,
-                              k_start, k_stop, 0, a, groups, xin, gather_src, act);
+        // Two-term activations of 16 rows take 2 x 16 x H bytes.  Where that fits LDS and an expert sees more than a
+        // few rows, one 8-wave block per CU keeps them resident; otherwise 2048-k windows and two 4-wave blocks per
+        // CU (the windows' barriers cost less than the lost second block when units are nearly empty, more when
+        // they are full: 32 tokens 125 / 130 us, 192 tokens 178 / 168 us at H 4096).
+        const size_t lds_res = b_lds_bytes<true, 0>(KT);
+        const bool resident = lds_res <= kLdsCap && (long)n * s.topk > 4L * s.n_experts && KT > kWindowKt;
+        if (resident) {
+            constexpr int W = GU_WAVES_RESIDENT_X2;
+            const int groups = (imax / 32 + W - 1) / W;
+            const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+            if ((rc = LdsLimit<&gate_up_mfma_kernel<W, true, 0>>::ensure(lds_res))) return rc;
+            hipExtLaunchKernelGGL((gate_up_mfma_kernel<W, true, 0>), dim3(blocks), dim3(W * 64), (uint32_t)lds_res, st,
+                                  k_start, k_stop, 0, a, groups, xin, gather_src, act);
+        } else {
+            const size_t lds = b_lds_bytes<true, kWindowKt>(KT);
+            const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
+            const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+            if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true, kWindowKt>>::ensure(lds))) return rc;
+            hipExtLaunchKernelGGL((gate_up_mfma_kernel<GU_WAVES, true, kWindowKt>), dim3(blocks), dim3(GU_WAVES * 64),
+                                  (uint32_t)lds, st, k_start, k_stop, 0, a, groups, xin, gather_src, act);
+        }
     } else {
-        if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false>>::ensure(lds))) return rc;
-        hipExtLaunchKernelGGL((gate_up_mfma_kernel<GU_WAVES, false>), dim3(blocks), dim3(GU_WAVES * 64), (uint32_t)lds, st,
+        const size_t lds = b_lds_bytes<false, 0>(KT);
+        const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
+        const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+        if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false, 0>>::ensure(lds))) return rc;
+        hipExtLaunchKernelGGL((gate_up_mfma_kernel<GU_WAVES, false, 0>), dim3(blocks), dim3(GU_WAVES * 64), (uint32_t)lds, st,
                               k_start, k_stop, 0, a, groups, xin, gather_src, act);
     }
     return check_launch("gate_up_mfma");
@@ -788,8 +901,8 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
         }
         return check_launch("down_prefill");
     }
-    if (units.unit_rows_cap != (x2 ? 8 : 16)) return FERRITE_ERR_INVALID_ARG;
-    const size_t lds = (size_t)a.act_ld * 16 + (size_t)((a.act_ld / 128 + 3) / 4) * 256;
+    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
+    const size_t lds = x2 ? b_lds_bytes<true, kWindowKt>(a.act_ld / 128) : b_lds_bytes<false, 0>(a.act_ld / 128);
     const int items = s.hidden / 64;
     const int groups = (items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW);
     const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
@@ -807,8 +920,9 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
 
 int warmup_experts_mfma() {
     int rc;
-    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false>>::ensure(kLdsCap))) return rc;
-    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false, 0>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true, kWindowKt>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES_RESIDENT_X2, true, 0>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES))) return rc;

@@ -84,9 +84,7 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     const int has_shared = s.shared_inter > 0;
     const size_t act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
     w.rows = (int)(nk + (has_shared ? n : 0));
-    // two-term activations: 8-row units (the two terms of a row share one 16-column operand)
-    w.unit_cap = mode == FERRITE_MODE_MFMA_FP8 ? unit_rows_for(n, s.topk, s.n_experts)
-                                               : (mode == FERRITE_MODE_MFMA_FP8_X2 ? 8 : 16);
+    w.unit_cap = mode == FERRITE_MODE_MFMA_FP8 ? unit_rows_for(n, s.topk, s.n_experts) : 16;
     w.max_units = max_units_for(n, s.topk, s.n_experts, has_shared, w.unit_cap);
     size_t off = 0;
     w.counters = bump(off, ((size_t)n + 1) * 4);   // first: ferrite_moe_layer_workspace_init clears it
@@ -419,19 +417,20 @@ extern "C" int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const fer
                                        ferrite_stream_t stream) {
     int rc = check_shape(shape, n, mode);
     if (rc) return rc;
-    if (!li || !blk || !out || !workspace || !blk->norm_w || !blk->residual || !blk->post || !blk->comb)
-        return FERRITE_ERR_INVALID_ARG;
-    if (blk->nh <= 0) return FERRITE_ERR_INVALID_ARG;
+    if (!li || !blk || !out || !workspace || !blk->norm_w) return FERRITE_ERR_INVALID_ARG;
+    const bool with_hc_post = blk->residual != nullptr;
+    if (with_hc_post && (!blk->post || !blk->comb || blk->nh <= 0)) return FERRITE_ERR_INVALID_ARG;
     const ferrite_moe_shape& s = *shape;
     const size_t layer_bytes = carve(s, n, mode).total, extra = block_extra(s, n);
     if (workspace_bytes < layer_bytes + 2 * extra) return FERRITE_ERR_WORKSPACE;
     char* b = static_cast<char*>(workspace);
     float* hfn = reinterpret_cast<float*>(b + layer_bytes);
-    float* ffn_out = reinterpret_cast<float*>(b + layer_bytes + extra);
+    float* ffn_out = with_hc_post ? reinterpret_cast<float*>(b + layer_bytes + extra) : out;
     if ((rc = ferrite_rmsnorm_f32(li, blk->norm_w, blk->eps, hfn, n, s.hidden, stream))) return rc;
     if ((rc = moe_layer_impl(shape, wts, packed, hfn, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
                              layer_bytes, stream, nullptr)))
         return rc;
+    if (!with_hc_post) return FERRITE_OK;
     return ferrite_hc_post_f32(ffn_out, blk->residual, blk->post, blk->comb, out, n, blk->nh, s.hidden, stream);
 }
 

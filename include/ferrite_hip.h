@@ -201,7 +201,7 @@ typedef struct ferrite_moe_workspace_view {
 
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
 /* Rows per unit (the token tile of the expert GEMMs) a layer call with these arguments uses: 16 = weights streamed
- * once per unit (decode-sized batches; 8 with two-term activations, whose two terms share the 16 operand columns),
+ * once per unit (decode-sized batches, any activation format),
  * 128 = both operands tiled through LDS (prefill-sized batches); 0 for an
  * unsupported shape.  The choice is a pure function of (shape, n, mode) and of the FERRITE_OVERRIDE_UNIT_ROWS
  * override, like the workspace layout that depends on it.
@@ -261,14 +261,16 @@ int ferrite_hc_post_f32(const float* x, const float* residual, const float* post
  *     hfn     = rmsnorm(li, post_attention_layernorm.weight, eps)
  *     ffn_out = moe_ffn(hfn)                       (ferrite_moe_layer_mxfp4 on f32 activations)
  *     out     = hc_post(ffn_out, residual, post, comb)
- * li [n, H] f32 (the mixed stream that hc_pre produced), out [n, nh, H] f32.  The workspace is the layer's followed by
+ * li [n, H] f32 (the mixed stream that hc_pre produced), out [n, nh, H] f32.  With residual == NULL the call ends
+ * after the second statement and out is ffn_out [n, H] (post, comb and nh are then ignored): the pre-norm layer
+ * without hyper-connections, which is also how consecutive layers are chained (out of one = li of the next).  The workspace is the layer's followed by
  * two [n, H] f32 buffers: size it with ferrite_moe_block_workspace_bytes and initialise it once with
  * ferrite_moe_layer_workspace_init (which only touches the layer's part).  Same rules as the layer call: no
  * allocation, no synchronisation, a launch sequence that depends only on (shape, n, mode), capturable. */
 typedef struct {
     const float* norm_w;    /* [H] */
     float eps;
-    const float* residual;  /* [n, nh, H] */
+    const float* residual;  /* [n, nh, H], or NULL: no hc_post */
     const float* post;      /* [n, nh] */
     const float* comb;      /* [n, nh, nh] */
     int nh;                 /* hyper-connection streams (hc_mult), <= 8 */

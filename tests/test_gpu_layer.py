@@ -88,7 +88,7 @@ def test_layer_c0_mfma_modes(hip, oracle, mode, key):
     out, v, _, _ = check_mfma(hip, oracle, layer, inp, mode)
     g = np.load(os.path.join(os.path.dirname(__file__), "golden", "c0_layer.npz"))
     assert max_abs_rel(out, g[key]) <= TOL_MFMA
-    assert hip.unit_rows(layer, inp.cfg.n, mode) == (8 if mode == MODE_MFMA_FP8_X2 else 16)
+    assert hip.unit_rows(layer, inp.cfg.n, mode) == 16
 
 
 def test_layer_smoke_fixture(hip, oracle):
@@ -104,8 +104,7 @@ def test_layer_smoke_fixture(hip, oracle):
 
 @pytest.mark.parametrize("seed,n", [(1, 1), (2, 3), (3, 17), (4, 40), (12, 90)])
 def test_layer_small_shapes_all_modes(hip, oracle, seed, n):
-    """Ragged token counts: units of 1..16 rows (1..8 with two-term activations), more than one unit per expert,
-    experts with no tokens."""
+    """Ragged token counts: units of 1..16 rows, more than one unit per expert, experts with no tokens."""
     cfg = synth.MoeConfig(n, 256, 8, 3, 256, 128, 4, 2)
     inp = synth.make_inputs(cfg, seed=seed)
     layer = hip.load_moe_layer(inp)
@@ -115,6 +114,19 @@ def test_layer_small_shapes_all_modes(hip, oracle, seed, n):
     assert max_abs_rel(out, ref32["out"]) <= TOL_F32
     check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8, ref32)
     check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8_X2, ref32)
+
+
+@pytest.mark.parametrize("n,hidden,inter,shared", [(24, 2304, 2304, 2304), (19, 2176, 128, 2432), (5, 4096, 256, 0)])
+def test_two_term_long_reductions_stream_their_activations_in_windows(hip, oracle, n, hidden, inter, shared):
+    """Two-term activations of a reduction longer than 2048 do not stay in LDS whole: they pass through a ring of
+    two 1024-k windows (gate/up when hidden > 2048, down when the intermediate size is).  Lengths that are not
+    multiples of the window, units of 1..16 rows, a shared expert whose size differs from the routed ones'."""
+    cfg = synth.MoeConfig(n, hidden, 8, 3, inter, shared, 4, 2)
+    inp = synth.make_inputs(cfg, seed=n)
+    layer = hip.load_moe_layer(inp)
+    ref32 = oracle.moe_ffn_mxfp4(inp, n_threads=8)
+    check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8_X2, ref32)
+    check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8, ref32)
 
 
 def test_two_term_mode_is_for_decode_sized_batches(hip):
@@ -254,7 +266,7 @@ def test_layer_all_tokens_on_the_same_experts(hip, oracle, n):
     assert v["counts"].max() == n and (v["counts"] > 0).sum() == 3
     assert max_abs_rel(out, ref32["out"]) <= TOL_F32
     check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8, ref32)
-    if n == 40:      # decode-sized: five full 8-row units per expert in the two-term mode
+    if n == 40:      # decode-sized: two full units and a ragged one per expert, two-term
         check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8_X2, ref32)
 
 
@@ -402,8 +414,7 @@ def test_layer_c2_prefill_scale(hip, oracle):
 
 @pytest.mark.parametrize("mode", [MODE_MFMA_FP8_X2, MODE_MFMA_FP8])
 def test_layer_c4_decode192(hip, oracle, mode):
-    """One layer of the 42-layer decode step: 192 tokens, about twelve rows per expert (two 8-row units with
-    two-term activations, one 16-row unit otherwise)."""
+    """One layer of the 42-layer decode step: 192 tokens, about twelve rows per expert."""
     _scale_check(hip, oracle, synth.CONFIGS["c4"], n_sample=12, mode=mode)
 
 
