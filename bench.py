@@ -34,7 +34,7 @@ MFMA_PEAK_FP4_TFLOPS = 10100.0 # dense MXFP4 x MXFP4
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
 # counters' reading for a 1 GiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw values
 # are in profiles/.  Counters cannot be read inside this script.
-MEASURED_TRAFFIC = {("c1", "gate_up_mfma_kernel"): 763.5e6, ("c2", "gate_up_prefill_kernel"): 1470.3e6}
+MEASURED_TRAFFIC = {("c1", "gate_up_mfma_kernel"): 764.6e6, ("c2", "gate_up_prefill_kernel"): 1470.3e6}
 
 WORKLOADS = {
     "c0": "c0: tiny parity layer, 8 tokens, H256 E16 top4 (4 groups/2) I128, MXFP4 weights, f32 activations",
