@@ -86,10 +86,12 @@ int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* 
 int check_routing_params(int e, int topk, int n_group, int topk_group);
 size_t perm_scratch_bytes(int n_tokens, int n_experts);   // masks + offsets of the three-phase permutation
 bool head_supported(int n, int H, int E);
+bool head_norm_supported(int n, int H, int E);   // ... with rmsnorm of the (f32) input fused in front
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
                     int n, float* logits, float* probs, float* ids_f32, int32_t* ids, const ActPlanes& xq,
                     int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
-                    int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, hipStream_t st);
+                    int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, const float* norm_w,
+                    float eps, hipStream_t st);
 int launch_router_chain(const void* x, int x_dtype, const float* router_t, int n, int H, int E, float* logits,
                         hipStream_t st);
 int launch_router_transpose(const float* w, int E, int H, float* dst, hipStream_t st);

@@ -221,9 +221,12 @@ static int mark(void* const* ev, int i, hipStream_t st) {
     return e == hipSuccess ? FERRITE_OK : hip_fail(e, "hipEventRecord");
 }
 
+// norm_w (may be NULL): x is the un-normalised f32 stream and the fused head applies rmsnorm(x, norm_w, norm_eps) to
+// it on the fly; only legal where fused_norm_ok() says so.
 static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts, const uint8_t* packed,
                           const void* x, int x_dtype, int n, void* out, int out_dtype, int mode, void* workspace,
-                          size_t workspace_bytes, ferrite_stream_t stream, void* const* ev) {
+                          size_t workspace_bytes, ferrite_stream_t stream, void* const* ev,
+                          const float* norm_w = nullptr, float norm_eps = 0.0f) {
     int rc = check_shape(shape, n, mode);
     if (rc) return rc;
     // the packed buffer carries the router weight (transposed); the checkpoint-layout one is read only without it
@@ -269,6 +272,9 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                      w.max_units};
     if ((rc = mark(ev, 0, st))) return rc;
     const bool fused_head = packed != nullptr && head_supported(n, s.hidden, s.n_experts);
+    if (norm_w && !(fused_head && is_mfma_mode(mode) && x_dtype == FERRITE_DT_F32 &&
+                    head_norm_supported(n, s.hidden, s.n_experts)))
+        return FERRITE_ERR_INVALID_ARG;
     if (fused_head) {
         // 1-3 (+ activation quantisation) as one launch
         PackedLayout L = packed_layout(s);
@@ -277,7 +283,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                                   n, logits, probs, ids_f32, ids, xq, reinterpret_cast<int32_t*>(b + w.counters),
                                   reinterpret_cast<int32_t*>(b + w.counts), reinterpret_cast<int32_t*>(b + w.starts),
                                   perm_map, gather_src, reinterpret_cast<int32_t*>(b + w.active),
-                                  reinterpret_cast<int32_t*>(b + w.n_active), &units, fuse_perm, st)))
+                                  reinterpret_cast<int32_t*>(b + w.n_active), &units, fuse_perm, norm_w, norm_eps, st)))
             return rc;
         if ((rc = mark(ev, 1, st))) return rc;
         if ((rc = mark(ev, 2, st))) return rc;
@@ -426,10 +432,18 @@ extern "C" int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const fer
     char* b = static_cast<char*>(workspace);
     float* hfn = reinterpret_cast<float*>(b + layer_bytes);
     float* ffn_out = with_hc_post ? reinterpret_cast<float*>(b + layer_bytes + extra) : out;
-    if ((rc = ferrite_rmsnorm_f32(li, blk->norm_w, blk->eps, hfn, n, s.hidden, stream))) return rc;
-    if ((rc = moe_layer_impl(shape, wts, packed, hfn, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
-                             layer_bytes, stream, nullptr)))
-        return rc;
+    // In the MFMA modes nothing but the fused head reads the normalised activations (the expert GEMMs take their
+    // quantised form, which the head writes), so the head normalises on the fly and hfn never exists in memory.
+    const bool fused_norm = is_mfma_mode(mode) && packed != nullptr && head_norm_supported(n, s.hidden, s.n_experts);
+    if (fused_norm) {
+        rc = moe_layer_impl(shape, wts, packed, li, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
+                            layer_bytes, stream, nullptr, blk->norm_w, blk->eps);
+    } else {
+        if ((rc = ferrite_rmsnorm_f32(li, blk->norm_w, blk->eps, hfn, n, s.hidden, stream))) return rc;
+        rc = moe_layer_impl(shape, wts, packed, hfn, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
+                            layer_bytes, stream, nullptr);
+    }
+    if (rc) return rc;
     if (!with_hc_post) return FERRITE_OK;
     return ferrite_hc_post_f32(ffn_out, blk->residual, blk->post, blk->comb, out, n, blk->nh, s.hidden, stream);
 }

@@ -563,6 +563,8 @@ struct HeadArgs {
     ActPlanes xq;         // q may be NULL: no quantisation blocks are launched then; q2 set: two-term
     int32_t* counters;    // [1 + n]
     int fuse_perm;        // the block that routes the last token also builds the permutation; else a separate launch does
+    const float* norm_w;  // not NULL: x is the un-normalised f32 stream and every block applies rmsnorm(x, norm_w, eps)
+    float eps;            // to its token(s) first (cpu.rs:124-143), so the normalised activations never go through HBM
     PermArgs perm;
 };
 
@@ -614,11 +616,83 @@ __device__ __forceinline__ void head_pmul(const HeadSet<T, W>& st, const float4*
     }
 }
 
+// rmsnorm of the block's token(s) in place of the first barrier ("x is in LDS") of every wave's role.  On entry
+// every thread has staged its share of the raw rows in xl and of their squares (each rounded once) in sq.  The
+// reference sums the squares of a row left to right in f32 (cpu.rs:124-143): a serial chain, walked by wave 0 with
+// 16-byte broadcast reads in counted batches, while the producer waves' first weight loads are already in flight.
+// Then all waves scale xl to (x * inv) * w, which is what the router chain and the quantisation see.
+struct HeadNorm {
+    const float* w;
+    float eps;
+    float4* xl;
+    const float4* sq;
+    float* inv;   // [T] in LDS
+    int nk4, T;
+};
+
+__device__ __forceinline__ float sumsq_chain(const float4* s4, int n4) {
+    float ss = 0.0f;
+    const int nb = n4 / 8;   // n4 is a multiple of 32
+    float4 r[2][8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[0][j] = s4[j];
+    for (int b = 0; b < nb; b += 2) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int bb = b + half;
+            if (bb < nb) {
+                if (bb + 1 < nb) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) r[half ^ 1][j] = s4[(bb + 1) * 8 + j];
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_waitcnt(0xC87F);   // lgkmcnt <= 8: everything but the batch just issued
+                } else {
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_waitcnt(0xC07F);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float4 p = r[half][j];
+                    ss = fadd(ss, p.x);
+                    ss = fadd(ss, p.y);
+                    ss = fadd(ss, p.z);
+                    ss = fadd(ss, p.w);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    return ss;
+}
+
+__device__ __forceinline__ void head_first_sync(const HeadNorm& nm) {
+    __syncthreads();   // x (and with a norm the squares) are in LDS
+    if (nm.w == nullptr) return;
+    const int tid = threadIdx.x;
+    if (tid < 64) {
+        for (int ti = 0; ti < nm.T; ++ti) {
+            float ss = sumsq_chain(nm.sq + (size_t)ti * nm.nk4, nm.nk4);
+            ss = fdiv(ss, (float)(nm.nk4 * 4));
+            const float inv = fdiv(1.0f, fsqrt(fadd(ss, nm.eps)));
+            if (tid == 0) nm.inv[ti] = inv;
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < nm.T * nm.nk4; i += blockDim.x) {
+        const int ti = i / nm.nk4, k4 = i - ti * nm.nk4;
+        const float iv = nm.inv[ti];
+        const float4 v = nm.xl[i], g = reinterpret_cast<const float4*>(nm.w)[k4];
+        nm.xl[i] = make_float4(fmul(fmul(v.x, iv), g.x), fmul(fmul(v.y, iv), g.y), fmul(fmul(v.z, iv), g.z),
+                               fmul(fmul(v.w, iv), g.w));
+    }
+    __syncthreads();   // the normalised rows are in place and the squares' space is free for the products
+}
+
 // Products of chunk c+1 are made while the chain consumes chunk c; register set c%4 holds the weights of chunk c
 // and is reloaded for chunk c+4 as soon as it has been used.
 template <int T, int W, int P>
 __device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int Epad, int nk4, const float4* xl,
-                                              float4* ring, int lane) {
+                                              float4* ring, int lane, const HeadNorm& nm) {
     constexpr int CH = HeadCfg<T, W>::CH;
     const int nch = nk4 / CH;
     float4* b0 = ring;
@@ -628,7 +702,7 @@ __device__ __forceinline__ void head_producer(const float4* __restrict__ wp, int
     head_pload<T, W, P>(s1, wp, Epad, 1, nch);
     head_pload<T, W, P>(s2, wp, Epad, 2, nch);
     head_pload<T, W, P>(s3, wp, Epad, 3, nch);
-    __syncthreads();   // x is in LDS
+    head_first_sync(nm);   // x is in LDS
     head_pmul<T, W, P>(s0, xl, nk4, 0, b0, lane);
     head_pload<T, W, P>(s0, wp, Epad, 4, nch);
     __syncthreads();
@@ -684,13 +758,13 @@ __device__ __forceinline__ void head_consume(float (&s)[T], const float4* buf, i
 
 // Barriers pair one to one with head_producer's.
 template <int T, int W>
-__device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const float4* ring, int lane) {
+__device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const float4* ring, int lane, const HeadNorm& nm) {
     constexpr int CH = HeadCfg<T, W>::CH;
     const int nch = nk4 / CH;
     const float4* b0 = ring;
     const float4* b1 = ring + CH * T * 64;
     __builtin_amdgcn_s_setprio(3);   // ahead of another block's producer waves on the same SIMD
-    __syncthreads();
+    head_first_sync(nm);
     __syncthreads();
     for (int c = 0; c < nch; c += 4) {
         head_consume<T, W>(s, b0, lane);
@@ -707,9 +781,9 @@ __device__ __forceinline__ void head_consumer(float (&s)[T], int nk4, const floa
 
 // The barriers of head_producer / head_consumer and nothing else.
 template <int T, int W>
-__device__ __forceinline__ void head_bystander(int nk4) {
+__device__ __forceinline__ void head_bystander(int nk4, const HeadNorm& nm) {
     const int nch = nk4 / HeadCfg<T, W>::CH;
-    __syncthreads();
+    head_first_sync(nm);
     __syncthreads();
     for (int c = 0; c < nch; c += 4) {
         __syncthreads();
@@ -732,6 +806,22 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
             const int t = t0 + ti;
             if (t >= a.n) break;
             const XT* xrow = static_cast<const XT*>(a.x) + (size_t)t * H;
+            if constexpr (sizeof(XT) == 4) {
+                if (a.norm_w) {
+                    // normalise the row in LDS first (the same three steps as in the logits blocks), quantise from there
+                    float4* row = reinterpret_cast<float4*>(head_lds + HeadCfg<T, W>::RING_BYTES);
+                    float4* sq = reinterpret_cast<float4*>(head_lds);
+                    float* inv = reinterpret_cast<float*>(head_lds + HeadCfg<T, W>::RING_BYTES + (size_t)T * H * 4);
+                    __syncthreads();   // the previous token's quantisation has read its row
+                    for (int i = tid; i < H / 4; i += 512) {
+                        const float4 v = reinterpret_cast<const float4*>(xrow)[i];
+                        row[i] = v;
+                        sq[i] = make_float4(fmul(v.x, v.x), fmul(v.y, v.y), fmul(v.z, v.z), fmul(v.w, v.w));
+                    }
+                    head_first_sync(HeadNorm{a.norm_w, a.eps, row, sq, inv, H / 4, 1});
+                    xrow = reinterpret_cast<const XT*>(row);
+                }
+            }
             for (int b = tid; b < H / 32; b += 512) {
                 const size_t at = (size_t)t * scale_pitch(H) + scale_pos(b), qo = (size_t)t * H + b * 32;
                 if (a.xq.q2) {
@@ -760,21 +850,26 @@ __global__ __launch_bounds__(512) void moe_head_kernel(HeadArgs a) {
             v = make_float4(u2f(q.x << 16), u2f(q.x & 0xffff0000u), u2f(q.y << 16), u2f(q.y & 0xffff0000u));
         }
         xl[i] = v;
+        if constexpr (sizeof(XT) == 4) {
+            if (a.norm_w) ring[i] = make_float4(fmul(v.x, v.x), fmul(v.y, v.y), fmul(v.z, v.z), fmul(v.w, v.w));
+        }
     }
+    const HeadNorm nm{sizeof(XT) == 4 ? a.norm_w : nullptr, a.eps, xl, ring,
+                      reinterpret_cast<float*>(head_lds + HeadCfg<T, W>::RING_BYTES + (size_t)T * H * 4), nk4, T};
     // wave 0 chains; wave 4 would share its SIMD (and its VALU issue slots) and only keeps the barriers company; the
     // others produce
     float s[T];
 #pragma unroll
     for (int ti = 0; ti < T; ++ti) s[ti] = 0.0f;
     switch (wave) {
-        case 0: head_consumer<T, W>(s, nk4, ring, lane); break;
-        case 1: head_producer<T, W, 0>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 2: head_producer<T, W, 1>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 3: head_producer<T, W, 2>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 5: head_producer<T, W, 3>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 6: head_producer<T, W, 4>(wp, a.Epad, nk4, xl, ring, lane); break;
-        case 7: head_producer<T, W, 5>(wp, a.Epad, nk4, xl, ring, lane); break;
-        default: head_bystander<T, W>(nk4); break;
+        case 0: head_consumer<T, W>(s, nk4, ring, lane, nm); break;
+        case 1: head_producer<T, W, 0>(wp, a.Epad, nk4, xl, ring, lane, nm); break;
+        case 2: head_producer<T, W, 1>(wp, a.Epad, nk4, xl, ring, lane, nm); break;
+        case 3: head_producer<T, W, 2>(wp, a.Epad, nk4, xl, ring, lane, nm); break;
+        case 5: head_producer<T, W, 3>(wp, a.Epad, nk4, xl, ring, lane, nm); break;
+        case 6: head_producer<T, W, 4>(wp, a.Epad, nk4, xl, ring, lane, nm); break;
+        case 7: head_producer<T, W, 5>(wp, a.Epad, nk4, xl, ring, lane, nm); break;
+        default: head_bystander<T, W>(nk4, nm); break;
     }
     // From here on wave 0 works alone (LDS is free for its scratch); with a fused permutation the other waves wait
     // at the barrier below and join in if this block turns out to be the one that routed the last token.
@@ -832,13 +927,20 @@ static HeadShape head_shape(int n, int eblocks) {
 
 static size_t head_lds_bytes(int n, int H, int E, bool fused) {
     const HeadShape hs = head_shape(n, (E + 63) / 64);
-    size_t b = 2 * (size_t)hs.W * 1024 + (size_t)hs.T * H * 4;
+    size_t b = 2 * (size_t)hs.W * 1024 + (size_t)hs.T * H * 4 + 64;   // ring, x rows, the rows' 1/rms
     if (fused) {
         if (b < sizeof(RouteScratch)) b = sizeof(RouteScratch);
         size_t p = perm_block_lds_bytes(n, E);
         if (p > b) b = p;
     }
     return b;
+}
+
+// The fused rmsnorm keeps the squares of the block's rows where the product ring will be.
+bool head_norm_supported(int n, int H, int E) {
+    if (!head_supported(n, H, E)) return false;
+    const HeadShape hs = head_shape(n, (E + 63) / 64);
+    return (size_t)hs.T * H * 4 <= 2 * (size_t)hs.W * 1024;
 }
 
 bool head_supported(int n, int H, int E) {
@@ -865,8 +967,10 @@ static int launch_head_t(const HeadArgs& a, int quant, size_t lds, hipStream_t s
 int launch_moe_head(const void* x, int x_dtype, const float* router_t, const float* bias, const ferrite_moe_shape& s,
                     int n, float* logits, float* probs, float* ids_f32, int32_t* ids, const ActPlanes& xq,
                     int32_t* counters, int32_t* counts, int32_t* starts, int32_t* perm_map, int32_t* gather_src,
-                    int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, hipStream_t st) {
+                    int32_t* active, int32_t* n_active, const UnitTables* units, int fuse_perm, const float* norm_w,
+                    float eps, hipStream_t st) {
     if (!head_supported(n, s.hidden, s.n_experts)) return FERRITE_DECLINED;
+    if (norm_w && (x_dtype != FERRITE_DT_F32 || !head_norm_supported(n, s.hidden, s.n_experts))) return FERRITE_DECLINED;
     HeadArgs a{};
     a.x = x; a.wt = router_t; a.bias = bias;
     a.n = n; a.H = s.hidden; a.E = s.n_experts; a.Epad = (s.n_experts + 63) / 64 * 64; a.topk = s.topk;
@@ -874,6 +978,7 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
     a.topk_group = s.topk_group; a.scaling = s.routed_scaling;
     a.logits = logits; a.probs = probs; a.ids_f32 = ids_f32; a.ids = ids; a.xq = xq; a.counters = counters;
     a.fuse_perm = fuse_perm;
+    a.norm_w = norm_w; a.eps = eps;
     PermArgs& p = a.perm;
     p.ids = ids; p.n = n; p.topk = s.topk; p.n_experts = s.n_experts;
     p.counts = counts; p.starts = starts; p.perm_map = perm_map; p.gather_src = gather_src;

@@ -376,11 +376,13 @@ def _block_oracle(oracle, inp, dc, li, norm_w, eps, residual, post, comb, act_mo
     return oracle.hc_post(ffn["out"], residual, post, comb), hfn
 
 
-@pytest.mark.parametrize("n", [8, 40])
-def test_block_rmsnorm_layer_hc_post(hip, oracle, n):
+@pytest.mark.parametrize("n,hidden,experts", [(8, 256, 16), (40, 256, 16), (150, 256, 16), (200, 384, 192), (300, 512, 64)])
+def test_block_rmsnorm_layer_hc_post(hip, oracle, n, hidden, experts):
     """exec/lib.rs:487-492 as one call: rmsnorm -> MoE FFN -> hc_post.  The normalised activations are bit-exact, so
-    routing is; the output keeps the layer's bars (relative to max|ref|)."""
-    cfg = synth.CONFIGS["c0"].with_tokens(n)
+    routing is; the output keeps the layer's bars (relative to max|ref|).  Sizes: every block shape of the fused
+    routing kernel (one token per block, two per block at 200 x 3 blocks of experts) and, at 300 tokens, the
+    separate launches, which take their rmsnorm as a launch of its own."""
+    cfg = synth.MoeConfig(n, hidden, experts, 4, 128, 128, 4, 2)
     inp, li, norm_w, residual, post, comb, dc = _block_case(cfg, seed=31)
     layer = hip.load_moe_layer(inp)
     d = lambda a: torch.from_numpy(a).to(hip.device)
@@ -390,6 +392,13 @@ def test_block_rmsnorm_layer_hc_post(hip, oracle, n):
         hip.sync()
         ref, hfn = _block_oracle(oracle, inp, dc, li, norm_w, 1e-6, residual, post, comb, act_mode)
         assert max_abs_rel(out.cpu().numpy(), ref) <= tol
+        # In the MFMA modes the normalised activations exist only inside the routing kernel (rmsnorm is fused into
+        # it); that they are the reference's, bit for bit, shows in the logits it leaves behind
+        v = hip.workspace_view(layer, n, mode, workspace=hip.block_workspace(layer, n, mode))
+        rr = oracle.moe_ffn_mxfp4(dc.replace(inp, x=hfn), act_mode=0, n_threads=8, want_out=False)
+        assert np.array_equal(v["logits"].cpu().numpy(), rr["logits"])
+        assert np.array_equal(v["ids"].cpu().numpy(), rr["ids"].astype(np.int32))
+        assert np.array_equal(v["probs"].cpu().numpy(), rr["probs"])
     # graph capture of the whole block, replayed on fresh data
     li_s, res_s = d(li).clone(), d(residual).clone()
     nw, po, co = d(norm_w), d(post), d(comb)
