@@ -145,10 +145,14 @@ __device__ __forceinline__ uint32_t combine_bf16(float f) {
 // A thread owns 16 bytes of every y row of its token (4 or 8 columns).  The slots are walked in batches of eight:
 // first the eight table entries, then the eight row pieces - all loads of a batch are in flight together - then the
 // products and sums in slot order.
+// With hc.residual set (f32 output only) the token's combined row x is not stored: the hyper-connection update that
+// follows the layer (KernelBackend::hc_post, cpu.rs:788-807) is applied to it in registers and its nh rows
+// out[t,i,:] = post[t,i] * x + sum_k comb[t,k,i] * residual[t,k,:] (k ascending, multiply and add rounded
+// separately) are what goes to memory.
 template <typename OT, typename YT>
 __global__ __launch_bounds__(256) void combine_kernel(const YT* __restrict__ y, const float* __restrict__ probs,
                                                       const int32_t* __restrict__ perm_map, int n, int topk,
-                                                      int H, int has_shared, OT* __restrict__ out) {
+                                                      int H, int has_shared, OT* __restrict__ out, HcPostArgs hc) {
     constexpr int N = YPiece<YT>::N;
     const int t = blockIdx.y;
     const int h = (blockIdx.x * blockDim.x + threadIdx.x) * N;
@@ -190,6 +194,32 @@ __global__ __launch_bounds__(256) void combine_kernel(const YT* __restrict__ y, 
     }
     OT* dst = out + (size_t)t * H + h;
     if constexpr (sizeof(OT) == 4) {
+        if (hc.residual != nullptr) {
+            const int nh = hc.nh;
+            for (int i = 0; i < nh; ++i) {
+                const float p = hc.post[(size_t)t * nh + i];
+                float acc[N];
+#pragma unroll
+                for (int c = 0; c < N; ++c) acc[c] = fmul(p, o[c]);
+                for (int k = 0; k < nh; ++k) {
+                    const float cf = hc.comb[((size_t)t * nh + k) * nh + i];
+                    const float* r = hc.residual + ((size_t)t * nh + k) * H + h;
+#pragma unroll
+                    for (int c = 0; c < N; c += 4) {
+                        const float4 rv = *reinterpret_cast<const float4*>(r + c);
+                        acc[c] = fadd(acc[c], fmul(cf, rv.x));
+                        acc[c + 1] = fadd(acc[c + 1], fmul(cf, rv.y));
+                        acc[c + 2] = fadd(acc[c + 2], fmul(cf, rv.z));
+                        acc[c + 3] = fadd(acc[c + 3], fmul(cf, rv.w));
+                    }
+                }
+                float* od = reinterpret_cast<float*>(out) + ((size_t)t * nh + i) * H + h;
+#pragma unroll
+                for (int c = 0; c < N; c += 4)
+                    *reinterpret_cast<float4*>(od + c) = make_float4(acc[c], acc[c + 1], acc[c + 2], acc[c + 3]);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < N; i += 4) *reinterpret_cast<float4*>(dst + i) = make_float4(o[i], o[i + 1], o[i + 2], o[i + 3]);
     } else {
@@ -219,20 +249,22 @@ int launch_down_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, co
 }
 
 int launch_combine(const void* y, int y_dtype, const float* probs, const int32_t* perm_map, int n, int topk,
-                   int hidden, int has_shared, void* out, int out_dtype, hipStream_t st) {
+                   int hidden, int has_shared, void* out, int out_dtype, hipStream_t st, const HcPostArgs* hcp) {
+    const HcPostArgs hc = hcp ? *hcp : HcPostArgs{nullptr, nullptr, nullptr, 0};
+    if (hc.residual && (out_dtype != FERRITE_DT_F32 || hc.nh < 1 || !hc.post || !hc.comb)) return FERRITE_ERR_INVALID_ARG;
     const bool of32 = out_dtype == FERRITE_DT_F32, yf32 = y_dtype == FERRITE_DT_F32;
     const int per_thread = yf32 ? 4 : 8;   // columns per thread: 16 bytes of a y row
     if (hidden % per_thread) return FERRITE_ERR_INVALID_ARG;
     dim3 grid((hidden / per_thread + 255) / 256, n);
     if ((!of32 && out_dtype != FERRITE_DT_BF16) || (!yf32 && y_dtype != FERRITE_DT_BF16)) return FERRITE_ERR_INVALID_ARG;
     if (of32 && yf32)
-        combine_kernel<float, float><<<grid, 256, 0, st>>>((const float*)y, probs, perm_map, n, topk, hidden, has_shared, (float*)out);
+        combine_kernel<float, float><<<grid, 256, 0, st>>>((const float*)y, probs, perm_map, n, topk, hidden, has_shared, (float*)out, hc);
     else if (of32)
-        combine_kernel<float, uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)y, probs, perm_map, n, topk, hidden, has_shared, (float*)out);
+        combine_kernel<float, uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)y, probs, perm_map, n, topk, hidden, has_shared, (float*)out, hc);
     else if (yf32)
-        combine_kernel<uint16_t, float><<<grid, 256, 0, st>>>((const float*)y, probs, perm_map, n, topk, hidden, has_shared, (uint16_t*)out);
+        combine_kernel<uint16_t, float><<<grid, 256, 0, st>>>((const float*)y, probs, perm_map, n, topk, hidden, has_shared, (uint16_t*)out, hc);
     else
-        combine_kernel<uint16_t, uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)y, probs, perm_map, n, topk, hidden, has_shared, (uint16_t*)out);
+        combine_kernel<uint16_t, uint16_t><<<grid, 256, 0, st>>>((const uint16_t*)y, probs, perm_map, n, topk, hidden, has_shared, (uint16_t*)out, hc);
     return check_launch("combine");
 }
 

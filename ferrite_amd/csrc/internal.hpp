@@ -102,8 +102,15 @@ int launch_gate_up_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w,
                        const int32_t* ids, const int32_t* gather_src, float* act, hipStream_t st);
 int launch_down_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, const float* act, int n,
                     const int32_t* ids, const int32_t* gather_src, float* y, hipStream_t st);
+// The hyper-connection update behind the layer, for a combine that applies it on the way out (f32 output only):
+// residual [n, nh, H], post [n, nh], comb [n, nh, nh]; out is then [n, nh, H].
+struct HcPostArgs {
+    const float *residual, *post, *comb;
+    int nh;
+};
 int launch_combine(const void* y, int y_dtype, const float* probs, const int32_t* perm_map, int n, int topk,
-                   int hidden, int has_shared, void* out, int out_dtype, hipStream_t st);
+                   int hidden, int has_shared, void* out, int out_dtype, hipStream_t st,
+                   const HcPostArgs* hc = nullptr);
 
 // experts_mfma.hip
 struct PackedLayout {

@@ -222,11 +222,12 @@ static int mark(void* const* ev, int i, hipStream_t st) {
 }
 
 // norm_w (may be NULL): x is the un-normalised f32 stream and the fused head applies rmsnorm(x, norm_w, norm_eps) to
-// it on the fly; only legal where fused_norm_ok() says so.
+// it on the fly; only legal where head_norm_supported() says so.  hc (may be NULL): the combine applies hc_post to
+// the layer's output on the way out; out is then [n, nh, H] f32.
 static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts, const uint8_t* packed,
                           const void* x, int x_dtype, int n, void* out, int out_dtype, int mode, void* workspace,
                           size_t workspace_bytes, ferrite_stream_t stream, void* const* ev,
-                          const float* norm_w = nullptr, float norm_eps = 0.0f) {
+                          const float* norm_w = nullptr, float norm_eps = 0.0f, const HcPostArgs* hc = nullptr) {
     int rc = check_shape(shape, n, mode);
     if (rc) return rc;
     // the packed buffer carries the router weight (transposed); the checkpoint-layout one is read only without it
@@ -344,7 +345,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     }
     if ((rc = mark(ev, 6, st))) return rc;
     // 6. weighted combine in slot order + shared expert (exec/lib.rs:1154-1164)
-    if ((rc = launch_combine(y, y_dtype, probs, perm_map, n, s.topk, s.hidden, has_shared, out, out_dtype, st))) return rc;
+    if ((rc = launch_combine(y, y_dtype, probs, perm_map, n, s.topk, s.hidden, has_shared, out, out_dtype, st, hc))) return rc;
     return mark(ev, 7, st);
 }
 
@@ -431,20 +432,23 @@ extern "C" int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const fer
     if (workspace_bytes < layer_bytes + 2 * extra) return FERRITE_ERR_WORKSPACE;
     char* b = static_cast<char*>(workspace);
     float* hfn = reinterpret_cast<float*>(b + layer_bytes);
-    float* ffn_out = with_hc_post ? reinterpret_cast<float*>(b + layer_bytes + extra) : out;
-    // In the MFMA modes nothing but the fused head reads the normalised activations (the expert GEMMs take their
-    // quantised form, which the head writes), so the head normalises on the fly and hfn never exists in memory.
+    // The two neighbours fold into the layer's own launches where nothing else needs their results in memory:
+    // rmsnorm into the fused routing head (MFMA modes: the expert GEMMs take the quantised activations that the head
+    // writes), hc_post into the combine (a per-element function of the layer's output).
     const bool fused_norm = is_mfma_mode(mode) && packed != nullptr && head_norm_supported(n, s.hidden, s.n_experts);
-    if (fused_norm) {
-        rc = moe_layer_impl(shape, wts, packed, li, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
-                            layer_bytes, stream, nullptr, blk->norm_w, blk->eps);
-    } else {
+    const bool fused_hc = with_hc_post && blk->nh <= 8 && (reinterpret_cast<uintptr_t>(blk->residual) & 15) == 0;
+    const HcPostArgs hc{blk->residual, blk->post, blk->comb, blk->nh};
+    float* ffn_out = (with_hc_post && !fused_hc) ? reinterpret_cast<float*>(b + layer_bytes + extra) : out;
+    const float* xin = li;
+    if (!fused_norm) {
         if ((rc = ferrite_rmsnorm_f32(li, blk->norm_w, blk->eps, hfn, n, s.hidden, stream))) return rc;
-        rc = moe_layer_impl(shape, wts, packed, hfn, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
-                            layer_bytes, stream, nullptr);
+        xin = hfn;
     }
-    if (rc) return rc;
-    if (!with_hc_post) return FERRITE_OK;
+    if ((rc = moe_layer_impl(shape, wts, packed, xin, FERRITE_DT_F32, n, ffn_out, FERRITE_DT_F32, mode, workspace,
+                             layer_bytes, stream, nullptr, fused_norm ? blk->norm_w : nullptr, blk->eps,
+                             fused_hc ? &hc : nullptr)))
+        return rc;
+    if (!with_hc_post || fused_hc) return FERRITE_OK;
     return ferrite_hc_post_f32(ffn_out, blk->residual, blk->post, blk->comb, out, n, blk->nh, s.hidden, stream);
 }
 

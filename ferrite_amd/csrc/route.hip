@@ -936,11 +936,14 @@ static size_t head_lds_bytes(int n, int H, int E, bool fused) {
     return b;
 }
 
-// The fused rmsnorm keeps the squares of the block's rows where the product ring will be.
+// The fused rmsnorm keeps the squares of the block's rows where the product ring will be.  Every block of a token
+// walks that token's sum-of-squares chain again, which pays while each block has a CU to itself (32 tokens, H 4096:
+// the block call 4 us shorter than with rmsnorm as a launch of its own) and no longer when two blocks share one
+// (192 tokens: 6 us longer): offered for the one-block-per-CU shape only.
 bool head_norm_supported(int n, int H, int E) {
     if (!head_supported(n, H, E)) return false;
     const HeadShape hs = head_shape(n, (E + 63) / 64);
-    return (size_t)hs.T * H * 4 <= 2 * (size_t)hs.W * 1024;
+    return hs.T == 1 && hs.W == 32 && (size_t)hs.T * H * 4 <= 2 * (size_t)hs.W * 1024;
 }
 
 bool head_supported(int n, int H, int E) {

@@ -379,9 +379,9 @@ def _block_oracle(oracle, inp, dc, li, norm_w, eps, residual, post, comb, act_mo
 @pytest.mark.parametrize("n,hidden,experts", [(8, 256, 16), (40, 256, 16), (150, 256, 16), (200, 384, 192), (300, 512, 64)])
 def test_block_rmsnorm_layer_hc_post(hip, oracle, n, hidden, experts):
     """exec/lib.rs:487-492 as one call: rmsnorm -> MoE FFN -> hc_post.  The normalised activations are bit-exact, so
-    routing is; the output keeps the layer's bars (relative to max|ref|).  Sizes: every block shape of the fused
-    routing kernel (one token per block, two per block at 200 x 3 blocks of experts) and, at 300 tokens, the
-    separate launches, which take their rmsnorm as a launch of its own."""
+    routing is; the output keeps the layer's bars (relative to max|ref|).  Up to 256 blocks of the fused routing
+    kernel (8, 40, 150 tokens here) rmsnorm runs inside it and hc_post inside the combine; beyond that, and with
+    the separate routing launches at 300 tokens, rmsnorm is a launch of its own."""
     cfg = synth.MoeConfig(n, hidden, experts, 4, 128, 128, 4, 2)
     inp, li, norm_w, residual, post, comb, dc = _block_case(cfg, seed=31)
     layer = hip.load_moe_layer(inp)
