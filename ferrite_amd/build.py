@@ -115,5 +115,8 @@ def build_host(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
+    if "--print-id" in sys.argv:   # what a binding bakes in to refuse a library of another build
+        print("ferrite-hip-" + source_hash())
+        sys.exit(0)
     print(build(verbose="-v" in sys.argv, incremental="--incremental" in sys.argv))
     print(build_host(verbose=True))

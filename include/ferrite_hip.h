@@ -121,8 +121,10 @@ int ferrite_act_quant_fp8(const void* x, int x_dtype, int64_t rows, int cols, ui
 
 /* The two-term form of ferrite_act_quant_fp8 that FERRITE_MODE_MFMA_FP8_X2 feeds the matrix cores with: q1 / scale1
  * as above, then q2 / scale2 = the same quantiser applied to the residual x - decode(q1) * scale1 (one f32
- * multiply by the power-of-two scale and one f32 subtraction per value).  No counterpart in the reference, whose
- * device path quantises once (dsv41_quant_fp8, crates/ferrite-models/src/dsv41/kernels.rs:97-108). */
+ * multiply by the power-of-two scale and one f32 subtraction per value).  The reference's e4m3 path quantises
+ * once (dsv41_quant_fp8, crates/ferrite-models/src/dsv41/kernels.rs:97-108); the decomposition itself is the one
+ * it applies to its e2m1 activations: out = x - dequant(q) * scale in f32, quantised again, both terms run
+ * against the same weight bytes (dsv41_sub_dequant_fp4, kernels/cuda/dsv41_kernels.cu:4138-4186). */
 int ferrite_act_quant_fp8_x2(const void* x, int x_dtype, int64_t rows, int cols, uint8_t* q1, uint8_t* scale1,
                              uint8_t* q2, uint8_t* scale2, ferrite_stream_t stream);
 

@@ -476,8 +476,10 @@ static void qdq_row_fp8(const float* x, int len, float* dst, uint8_t* tmpq, floa
 }
 
 /* Two-term form: q1/s1 = act_quant_fp8(x), q2/s2 = act_quant_fp8(x - decode(q1)*s1): x ~ dq1 + dq2.
- * Not in the reference (its device path quantises once, kernels.rs:97-108): the composition of its quantiser with
- * one f32 subtraction, stated here so that the device's two-term mode has a bit-level definition. */
+ * The reference's e4m3 path quantises once (kernels.rs:97-108); the residual step is the one it uses for its e2m1
+ * activations (out[i] = x[i] - decode(q[i]) * scale in f32, then the quantiser again: sub_dequant_fp4_kernel,
+ * kernels/cuda/dsv41_kernels.cu:4165-4179), stated here with the e4m3 quantiser so that the device's two-term mode
+ * has a bit-level definition. */
 void fo_act_quant_fp8_x2(const float* x, size_t len, uint8_t* q1, float* s1, uint8_t* q2, float* s2) {
     float* r = (float*)malloc(sizeof(float) * len);
     fo_act_quant_fp8(x, len, 32, 1, q1, s1);
