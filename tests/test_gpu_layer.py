@@ -380,8 +380,9 @@ def _block_oracle(oracle, inp, dc, li, norm_w, eps, residual, post, comb, act_mo
 def test_block_rmsnorm_layer_hc_post(hip, oracle, n, hidden, experts):
     """exec/lib.rs:487-492 as one call: rmsnorm -> MoE FFN -> hc_post.  The normalised activations are bit-exact, so
     routing is; the output keeps the layer's bars (relative to max|ref|).  Up to 256 blocks of the fused routing
-    kernel (8, 40, 150 tokens here) rmsnorm runs inside it and hc_post inside the combine; beyond that, and with
-    the separate routing launches at 300 tokens, rmsnorm is a launch of its own."""
+    kernel (8, 40, 150 tokens here) rmsnorm runs inside it; beyond that, and with the separate routing launches at
+    300 tokens, rmsnorm is a launch of its own.  hc_post runs inside the combine up to 256 tokens, as its own
+    launch at 300."""
     cfg = synth.MoeConfig(n, hidden, experts, 4, 128, 128, 4, 2)
     inp, li, norm_w, residual, post, comb, dc = _block_case(cfg, seed=31)
     layer = hip.load_moe_layer(inp)
