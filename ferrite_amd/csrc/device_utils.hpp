@@ -115,4 +115,55 @@ __device__ __forceinline__ uint32_t quant_block32_x2(const XT* __restrict__ src,
     return s1 | (s2 << 8);
 }
 
+// The left-to-right f32 sum (separately rounded adds, the reference's rmsnorm order: cpu.rs:124-143) of the n4
+// float4 at s4 in LDS, continued from ss.  Every lane reads the same addresses and holds the same running sum.
+// Straight-line pieces of eight batches (256 values): a batch of eight 16-byte reads is in flight while the 32
+// dependent adds of the batch before it run, and nothing is in flight at the end of a piece.  With the two
+// register buffers carried around a loop instead, the compiler copied one buffer into the other every iteration and
+// waited for every outstanding read at the top of a batch: 15 us for 4096 values against 10 us this way.
+__device__ __forceinline__ float sumsq_piece(const float4* p, float ss) {
+    constexpr int NB = 8;
+    float4 r[2][8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) r[0][j] = p[j];
+#pragma unroll
+    for (int g = 0; g < NB; ++g) {
+        if (g + 1 < NB) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) r[(g + 1) & 1][j] = p[(g + 1) * 8 + j];
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xC87F);   // lgkmcnt <= 8: everything but the batch just issued
+        } else {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float4 q = r[g & 1][j];
+            ss = fadd(ss, q.x);
+            ss = fadd(ss, q.y);
+            ss = fadd(ss, q.z);
+            ss = fadd(ss, q.w);
+        }
+        // pins the batch's adds in front of the next batch's reads (the optimiser otherwise hoists all 64 reads of
+        // the piece to its top, 256 registers) and the reads behind it
+        asm volatile("" : "+v"(ss) : : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    return ss;
+}
+
+__device__ __forceinline__ float sumsq_walk(const float4* s4, int n4, float ss) {
+    const int pieces = n4 >> 6;
+    for (int i = 0; i < pieces; ++i) ss = sumsq_piece(s4 + i * 64, ss);
+    for (int j = pieces * 64; j < n4; ++j) {
+        const float4 q = s4[j];
+        ss = fadd(ss, q.x);
+        ss = fadd(ss, q.y);
+        ss = fadd(ss, q.z);
+        ss = fadd(ss, q.w);
+    }
+    return ss;
+}
+
 }  // namespace fe

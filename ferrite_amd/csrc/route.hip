@@ -630,48 +630,13 @@ struct HeadNorm {
     int nk4, T;
 };
 
-__device__ __forceinline__ float sumsq_chain(const float4* s4, int n4) {
-    float ss = 0.0f;
-    const int nb = n4 / 8;   // n4 is a multiple of 32
-    float4 r[2][8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) r[0][j] = s4[j];
-    for (int b = 0; b < nb; b += 2) {
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const int bb = b + half;
-            if (bb < nb) {
-                if (bb + 1 < nb) {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) r[half ^ 1][j] = s4[(bb + 1) * 8 + j];
-                    __builtin_amdgcn_sched_barrier(0);
-                    __builtin_amdgcn_s_waitcnt(0xC87F);   // lgkmcnt <= 8: everything but the batch just issued
-                } else {
-                    __builtin_amdgcn_sched_barrier(0);
-                    __builtin_amdgcn_s_waitcnt(0xC07F);
-                }
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float4 p = r[half][j];
-                    ss = fadd(ss, p.x);
-                    ss = fadd(ss, p.y);
-                    ss = fadd(ss, p.z);
-                    ss = fadd(ss, p.w);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    }
-    return ss;
-}
-
 __device__ __forceinline__ void head_first_sync(const HeadNorm& nm) {
     __syncthreads();   // x (and with a norm the squares) are in LDS
     if (nm.w == nullptr) return;
     const int tid = threadIdx.x;
     if (tid < 64) {
         for (int ti = 0; ti < nm.T; ++ti) {
-            float ss = sumsq_chain(nm.sq + (size_t)ti * nm.nk4, nm.nk4);
+            float ss = sumsq_walk(nm.sq + (size_t)ti * nm.nk4, nm.nk4, 0.0f);
             ss = fdiv(ss, (float)(nm.nk4 * 4));
             const float inv = fdiv(1.0f, fsqrt(fadd(ss, nm.eps)));
             if (tid == 0) nm.inv[ti] = inv;
