@@ -307,7 +307,7 @@ def test_pack_is_a_pure_permutation(hip, oracle):
 
 
 # ---- the steps before and after the layer ----
-@pytest.mark.parametrize("n,dim", [(1, 4), (11, 4096), (3, 517), (5, 7168), (2, 9000)])
+@pytest.mark.parametrize("n,dim", [(1, 4), (11, 4096), (3, 517), (5, 7168), (2, 9000), (3, 520), (7, 1028), (1500, 256)])
 def test_rmsnorm_bit_exact_vs_oracle(hip, oracle, n, dim):  # gpu_smoke.rs:56-70 shape [11, 4096] included
     rng = np.random.default_rng(n * 1000 + dim)
     x = (rng.standard_normal((n, dim)) * rng.uniform(1e-3, 30, (n, 1))).astype(np.float32)
