@@ -26,6 +26,11 @@ typedef unsigned int u4v __attribute__((ext_vector_type(4)));  // 128-bit vector
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Which main loop the 128-row units run on (a test hook, ferrite_hip_set_override): 0 = both operands staged
+// through LDS, 1 / 2 = weights streamed into registers by blocks of 4 / 8 waves.
+static std::atomic<int> g_prefill_variant{0};
+void set_prefill_variant(int v) { g_prefill_variant.store(v, std::memory_order_relaxed); }
+
 PackedLayout packed_layout(const ferrite_moe_shape& s) {
     PackedLayout L{};
     const size_t H = s.hidden, I = s.inter, Is = s.shared_inter, E = s.n_experts;
@@ -328,7 +333,9 @@ struct MfmaArgs {
     const uint8_t* sh_scales;
     size_t codes_per_expert, scales_per_expert;
     const int32_t *unit_expert, *unit_row0, *unit_rows, *unit_first, *unit_count, *n_units;
+    const int32_t* unit_range;   // [lo, hi): the units this launch covers; NULL = all
     int n, topk, n_experts, hidden, inter, shared_inter, act_ld, unit_cap, max_units;
+    int n_early, dense_row0;     // experts [0, n_early): gate/up results in dense rows dense_row0 + expert * n + token
     float limit;
 };
 
@@ -348,16 +355,22 @@ __device__ __forceinline__ bool unit_ok(const MfmaArgs& a, int e, int row0, int 
 // Used by the 128-row kernels (2-3 units per expert) and by the 16-row kernels (the shared expert's n/16 units, an
 // expert with more than 16 rows).  Returns false for blocks without work or with inconsistent tables.
 __device__ __forceinline__ bool unit_block_work(const MfmaArgs& a, int groups, int& u, int& ig, int& ne) {
-    const int n_units = min(*a.n_units, a.max_units);
+    int lo = 0, hi = min(*a.n_units, a.max_units);
+    if (a.unit_range) {
+        lo = max(a.unit_range[0], 0);
+        hi = min(a.unit_range[1], hi);
+    }
+    const int n_units = hi - lo;
+    if (n_units <= 0) return false;
     const int total = n_units * groups, per_xcd = (total + 7) >> 3;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int v = xcd * per_xcd + slot;
     if (slot >= per_xcd || v >= total) return false;
-    const int up = v / groups;                       // some unit of the expert whose segment holds v
+    const int up = lo + v / groups;                  // some unit of the expert whose segment holds v
     const int first = a.unit_first[up];
     ne = a.unit_count[up];
-    if (first < 0 || ne < 1 || up < first || up >= first + ne || first + ne > n_units) return false;
-    const int vl = v - first * groups;               // 0 .. ne * groups - 1
+    if (first < lo || ne < 1 || up < first || up >= first + ne || first + ne > hi) return false;
+    const int vl = v - (first - lo) * groups;        // 0 .. ne * groups - 1
     ig = vl / ne;
     u = first + (vl - ig * ne);
     return true;
@@ -366,24 +379,15 @@ __device__ __forceinline__ bool unit_block_work(const MfmaArgs& a, int groups, i
 // gate/up GEMM + clamped SwiGLU + e4m3-per-32 quantisation of the result (one or two terms).
 // grid: unit_block_work over groups = ceil(items / WAVES) item groups; wave w of item group ig owns item
 // ig*WAVES + w of the unit's expert.
-template <int WAVES, bool kKeep, bool kX2, int WIN>
-__device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& xin,
-                                             const int32_t* __restrict__ gather_src, const ActPlanes& act,
-                                             unsigned char* lds_raw) {
-    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
-    if (!unit_ok(a, e, row0, nrows)) return;   // tables from an uninitialised workspace must not cause a fault
+// The unit (expert e, activation rows row0 .. row0 + nrows - 1, whose tokens row_src(c) names) against item group ig.
+template <int WAVES, bool kKeep, bool kX2, int WIN, typename RowFn>
+__device__ __forceinline__ void gate_up_rows(const MfmaArgs& a, int e, int row0, int nrows, int ig, RowFn row_src,
+                                             const ActPlanes& xin, const ActPlanes& act, unsigned char* lds_raw) {
     const bool shared = e == a.n_experts;
     const int inter = shared ? a.shared_inter : a.inter;
     const int items = inter / 32;
     if (ig * WAVES >= items) return;
     const int H = a.hidden, KT = H / 128, KT4 = (KT + 3) / 4;
-    const int nk = a.n * a.topk, topk = a.topk;
-    auto row_src = [&](int c) -> int {
-        int g = row0 + c;
-        if (shared) return g - nk;
-        int i = gather_src[g];
-        return (i < 0 || i >= nk) ? -1 : i / topk;
-    };
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int item = ig * WAVES + wave;
     const bool live = item < items;
@@ -449,6 +453,25 @@ __device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, c
         regs, lds_raw, lane);
 }
 
+template <int WAVES, bool kKeep, bool kX2, int WIN>
+__device__ __forceinline__ void gate_up_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& xin,
+                                             const int32_t* __restrict__ gather_src, const ActPlanes& act,
+                                             unsigned char* lds_raw) {
+    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    if (!unit_ok(a, e, row0, nrows)) return;   // tables from an uninitialised workspace must not cause a fault
+    const bool shared = e == a.n_experts;
+    const int nk = a.n * a.topk, topk = a.topk;
+    gate_up_rows<WAVES, kKeep, kX2, WIN>(
+        a, e, row0, nrows, ig,
+        [&](int c) -> int {
+            int g = row0 + c;
+            if (shared) return g - nk;
+            int i = gather_src[g];
+            return (i < 0 || i >= nk) ? -1 : i / topk;
+        },
+        xin, act, lds_raw);
+}
+
 // WIN: window of the activation staging in k steps, 0 = resident (see window_kt).  One-term activations are always
 // resident; two-term ones are windowed at 2048 k with two 4-wave blocks per CU, or resident with one 8-wave block
 // per CU (the launcher chooses).
@@ -464,10 +487,38 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gate_up_mfma_k
     else gate_up_unit<WAVES, false, kX2, WIN>(a, u, ig, xin, gather_src, act, lds_raw);
 }
 
+// gate/up of the experts [0, n_early) and of the shared expert for EVERY token, which needs nothing the router
+// produces: it runs beside the routing kernel (whose serial chain leaves HBM idle) and writes dense rows
+// dense_row0 + expert * n + token (the shared expert: its usual rows n * topk + token).  Units are (expert, 16
+// consecutive tokens); blocks map to (expert, item group, token tile) in the XCD-contiguous order of
+// unit_block_work, so the token tiles of one expert read its weights from one L2.  Per token the arithmetic is that
+// of the routed kernel (an MFMA column does not see its neighbours): the same bits.
+template <int WAVES, bool kX2, int WIN>
+__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gate_up_early_kernel(MfmaArgs a, int groups, ActPlanes xin,
+                                                                                       ActPlanes act) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    const int tiles = (a.n + 15) >> 4;
+    const int experts = a.n_early + (a.shared_inter > 0 ? 1 : 0);
+    const int total = experts * tiles * groups, per_xcd = (total + 7) >> 3;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int v = xcd * per_xcd + slot;
+    if (slot >= per_xcd || v >= total) return;
+    const int ee = v / (groups * tiles), r = v - ee * (groups * tiles);
+    const int ig = r / tiles, tile = r - ig * tiles;
+    const bool shared = ee >= a.n_early;
+    const int e = shared ? a.n_experts : ee;
+    const int t0 = tile * 16, nrows = min(16, a.n - t0);
+    const int row0 = (shared ? a.n * a.topk : a.dense_row0 + ee * a.n) + t0;
+    auto row_src = [&](int c) -> int { return t0 + c; };
+    if (tiles > 1) gate_up_rows<WAVES, true, kX2, WIN>(a, e, row0, nrows, ig, row_src, xin, act, lds_raw);
+    else gate_up_rows<WAVES, false, kX2, WIN>(a, e, row0, nrows, ig, row_src, xin, act, lds_raw);
+}
+
 // down GEMM: y[row][h] for the unit's rows.  grid: unit_block_work over groups = ceil(items / (WAVES*IPW)); item =
 // 64 rows of H.
 template <int WAVES, int IPW, bool kKeep, bool kX2>
-__device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& act, float* __restrict__ y,
+__device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& act,
+                                          const int32_t* __restrict__ gather_src, float* __restrict__ y,
                                           unsigned char* lds_raw) {
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
@@ -488,8 +539,17 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
     // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
     const BSource<kX2> bsrc{act, (size_t)a.act_ld, scale_pitch(a.act_ld), nrows};
     const int c = lane & 15, g = lane >> 4;
+    // an expert whose gate/up ran ahead of routing keeps its activations in dense rows, one per token
+    const bool dense = e < a.n_early;
+    const int nk = a.n * a.topk, dense0 = a.dense_row0 + e * a.n;
     run_unit<kKeep, kX2, kX2 ? kWindowKt : 0>(
-        bsrc, [&](int col) { return row0 + col; }, KT, IPW,
+        bsrc,
+        [&](int col) -> int {
+            if (!dense) return row0 + col;
+            const int i = gather_src[row0 + col];
+            return (i < 0 || i >= nk) ? -1 : dense0 + i / a.topk;
+        },
+        KT, IPW,
         [&](int r, const u4v*& wp, const u4v*& sp) {
             const int item = item0 + r;
             wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
@@ -509,12 +569,13 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
 
 template <int WAVES, int IPW, bool kX2>
 __global__ __launch_bounds__(WAVES * 64, 2) void down_mfma_kernel(MfmaArgs a, int groups, ActPlanes act,
+                                                               const int32_t* __restrict__ gather_src,
                                                                float* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig, ne;
     if (!unit_block_work(a, groups, u, ig, ne)) return;
-    if (ne > 1) down_unit<WAVES, IPW, true, kX2>(a, u, ig, act, y, lds_raw);
-    else down_unit<WAVES, IPW, false, kX2>(a, u, ig, act, y, lds_raw);
+    if (ne > 1) down_unit<WAVES, IPW, true, kX2>(a, u, ig, act, gather_src, y, lds_raw);
+    else down_unit<WAVES, IPW, false, kX2>(a, u, ig, act, gather_src, y, lds_raw);
 }
 
 
@@ -802,6 +863,324 @@ __global__ __launch_bounds__(PF_WAVES * 64, PF_WAVES == 4 ? 2 : 1) void down_pre
     }
 }
 
+// ---- prefill kernels, weight-streaming form --------------------------------------------------------------
+// One block (W waves) computes W items x NT*16 grouped rows of one unit.  Wave w owns item w for all of the rows:
+// its weights go from global memory straight into registers, 16 bytes per lane and tile as in the 16-row kernels,
+// through a ring of three k steps, so that a k step's tiles were asked for two to three steps before they are
+// used: far enough ahead for HBM.  Only the activations are shared by the block's waves and go through LDS: a ring
+// of three stages of one k step each ([tile][half][64 lanes] 16-byte slots in the operand order and slot swizzle
+// of the LDS-staged kernels, then [tile][64 lanes] scale words), filled through registers (ordinary loads keep the
+// compiler's wait counts exact, which loads that write LDS directly do not): the loads of step k+2 are issued at
+// the top of step k, written to their stage at the top of step k+1 and read during step k+2, one barrier per step.
+// Accumulation order over k is that of the other kernels: the same bits.
+template <int W, int NT>
+struct StCfg {
+    static constexpr int STAGES = 3;
+    static constexpr int CODE_SLOTS = NT * 128;            // 16-byte slots of e4m3 codes per stage
+    static constexpr int STAGE_SLOTS = CODE_SLOTS + NT * 16;   // + NT * 64 scale words
+    static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_SLOTS * 16;
+    static constexpr int CF = 2 * NT / W;                  // 1 KiB pieces of codes per wave and stage
+    static constexpr int SF = (NT + W - 1) / W;            // 256-byte pieces of scale words per wave and stage
+    static_assert((2 * NT) % W == 0, "the code pieces of a stage must divide among the waves");
+};
+
+// All four streams of a block are read through buffer resources (a wave-uniform base in scalar registers, a 32-bit
+// byte offset per lane that does not change over k, and the k step as a scalar offset): no 64-bit address
+// arithmetic in vector registers, of which this kernel has none to spare, and reads past a stream's end return 0.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(bytes > 0xffffffffull ? 0xffffffffull : bytes),
+                                             0x00020000);
+}
+__device__ __forceinline__ u4v rsrc_ld16(rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+}
+__device__ __forceinline__ uint32_t rsrc_ld4(rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0);
+}
+
+template <int W, int NT>
+struct StCtx {
+    rsrc_t ra, ras;          // this wave's item: codes [KT][4 tiles][64 lanes][16 B], scale words [KT4][64 lanes][16 B]
+    rsrc_t rb, rbs;          // activation codes and scale rows (operand order)
+    uint32_t aoff;           // 16 * lane
+    uint32_t coff[StCfg<W, NT>::CF];   // byte offset of the lane's chunk of piece i at k step 0
+    uint32_t soff[StCfg<W, NT>::SF];   // byte offset of the lane's scale word of piece i, group 0
+    int KT, lane, wave, ntile, bslot;
+};
+
+// row_q(col) / row_s(col): byte offsets of unit column col's code row / scale row from bq / bs.
+template <int W, int NT, typename RowQ, typename RowS>
+__device__ __forceinline__ void st_context(StCtx<W, NT>& c, const uint8_t* cbase, const uint8_t* sbase, int item, int KT,
+                                           int nrows, const uint8_t* bq, size_t bq_bytes, const uint8_t* bs,
+                                           size_t bs_bytes, RowQ row_q, RowS row_s) {
+    using Cfg = StCfg<W, NT>;
+    const int KT4 = (KT + 3) >> 2;
+    c.KT = KT;
+    c.lane = threadIdx.x & 63;
+    c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    c.ntile = min(NT, (nrows + 15) >> 4);
+    c.ra = make_rsrc(cbase + (size_t)item * KT * 4096, (size_t)KT * 4096);
+    c.ras = make_rsrc(sbase + (size_t)item * KT4 * 1024, (size_t)KT4 * 1024);
+    c.rb = make_rsrc(bq, bq_bytes);
+    c.rbs = make_rsrc(bs, bs_bytes);
+    c.aoff = (uint32_t)c.lane * 16;
+    const int cc = c.lane & 15, g = c.lane >> 4;
+    // piece j of a stage = (tile j/2, half j%2): the four lanes of a quad fetch 64 consecutive bytes of row lane/4 of
+    // the tile, the chunk a lane fetches XORed with (row/2)%4 (see pf_context)
+#pragma unroll
+    for (int i = 0; i < Cfg::CF; ++i) {
+        const int j = c.wave * Cfg::CF + i;
+        const int col = (j >> 1) * 16 + (c.lane >> 2);
+        c.coff[i] = row_q(col < nrows ? col : 0) + (uint32_t)((j & 1) * 64 + ((c.lane & 3) ^ ((c.lane >> 3) & 3)) * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::SF; ++i) {
+        const int col = min(c.wave * Cfg::SF + i, NT - 1) * 16 + cc;
+        c.soff[i] = row_s(col < nrows ? col : 0) + (uint32_t)(g * 4);
+    }
+    c.bslot = 4 * cc + (g ^ ((cc >> 1) & 3));
+}
+
+template <int W, int NT>
+struct StFill {
+    u4v cr[StCfg<W, NT>::CF];
+    uint32_t sr[StCfg<W, NT>::SF];
+};
+
+template <int W, int NT>
+__device__ __forceinline__ void st_load(const StCtx<W, NT>& c, int kt, StFill<W, NT>& f) {
+#pragma unroll
+    for (int i = 0; i < StCfg<W, NT>::CF; ++i) f.cr[i] = rsrc_ld16(c.rb, c.coff[i], (uint32_t)kt * 128);
+#pragma unroll
+    for (int i = 0; i < StCfg<W, NT>::SF; ++i) f.sr[i] = rsrc_ld4(c.rbs, c.soff[i], (uint32_t)(kt >> 2) * 16);
+}
+
+template <int W, int NT>
+__device__ __forceinline__ void st_store(const StCtx<W, NT>& c, u4v* stage, const StFill<W, NT>& f) {
+    using Cfg = StCfg<W, NT>;
+#pragma unroll
+    for (int i = 0; i < Cfg::CF; ++i) stage[(c.wave * Cfg::CF + i) * 64 + c.lane] = f.cr[i];
+    uint32_t* sw = reinterpret_cast<uint32_t*>(stage + Cfg::CODE_SLOTS);
+#pragma unroll
+    for (int i = 0; i < Cfg::SF; ++i)
+        if (c.wave * Cfg::SF + i < NT) sw[(c.wave * Cfg::SF + i) * 64 + c.lane] = f.sr[i];
+}
+
+// The weights of k step kt (4 tiles) and the scale words of its group of four k steps.
+struct StWeights {
+    u4v a[4];
+    u4v sc;
+};
+
+template <int W, int NT>
+__device__ __forceinline__ void st_load_a(const StCtx<W, NT>& c, int kt, StWeights& w) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) w.a[t] = rsrc_ld16(c.ra, c.aoff + t * 1024, (uint32_t)kt * 4096);
+    w.sc = rsrc_ld16(c.ras, c.aoff, (uint32_t)(kt >> 2) * 1024);
+}
+
+// k step kt against stage R = kt % 3 of the ring, with the weights in ring slot R.  The scale operands select their
+// byte with op_sel 0: the words are shifted by the k step's byte (kt % 4) first, which leaves the unrolling free
+// to follow the rings.  Every load is issued whatever kt is (past the end the last k step is fetched again and never
+// used): a load behind a branch makes the compiler wait for all loads at the next use of any.
+// kFull: all NT tiles of rows are live; otherwise tiles beyond ntile get no MFMAs (a unit's last block of rows is
+// usually far from full).
+template <int R, bool kFull, int W, int NT>
+__device__ __forceinline__ void st_step(const StCtx<W, NT>& c, u4v* lds, int kt, StWeights (&w)[3], StFill<W, NT>& f,
+                                        v4f (&acc)[4][NT]) {
+    using Cfg = StCfg<W, NT>;
+    __syncthreads();   // stage R is complete; nobody reads the stage that is written next any more
+    st_store(c, lds + ((R + 1) % 3) * Cfg::STAGE_SLOTS, f);
+    __builtin_amdgcn_sched_barrier(0);
+    st_load(c, min(kt + 2, c.KT - 1), f);
+    __builtin_amdgcn_sched_barrier(0);
+    const u4v* stage = lds + R * Cfg::STAGE_SLOTS;
+    const uint32_t* sw = reinterpret_cast<const uint32_t*>(stage + Cfg::CODE_SLOTS);
+    const int sh = (kt & 3) * 8;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) w[R].sc[t] >>= sh;   // in place: a slot's scale words are used by this step only
+    // operand registers of the row tiles: two sets used in turn (a tile is read while the MFMAs of the tile before
+    // it run), or one where registers are short (the other wave of the SIMD then covers the read)
+    constexpr int NB = W * NT <= 32 ? 1 : 2;
+    u4v b[NB][2];
+    uint32_t bs[NB];
+    auto read_tile = [&](int tt) {
+        const u4v* bt = stage + tt * 128 + c.bslot;
+        b[tt % NB][0] = bt[0];
+        b[tt % NB][1] = bt[64];
+        bs[tt % NB] = sw[tt * 64 + c.lane];
+    };
+    read_tile(0);
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+        if (kFull || tt < c.ntile) {   // block-uniform
+            if (NB == 2 && tt + 1 < NT) read_tile(tt + 1);
+            const u4v b0 = b[tt % NB][0], b1 = b[tt % NB][1];
+            bs[tt % NB] >>= sh;
+            const v8i bv = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const v8i a8 = {(int)w[R].a[t][0], (int)w[R].a[t][1], (int)w[R].a[t][2], (int)w[R].a[t][3], 0, 0, 0, 0};
+                acc[t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, bv, acc[t][tt], 4 /*A e2m1*/, 0 /*B e4m3*/,
+                                                                              0, (int)w[R].sc[t], 0, (int)bs[tt % NB]);
+            }
+            if (NB == 1 && tt + 1 < NT) read_tile(tt + 1);
+            // Pins the tile: its MFMAs stay in front of this point and the operand reads of the tiles after the next
+            // behind it.  Without it the compiler reads all tiles of the step first (64 more registers than there are).
+            if constexpr (NT * 16 > 128)   // 256 accumulators live in the accumulation registers
+                asm volatile("" : "+a"(acc[0][tt]), "+a"(acc[1][tt]), "+a"(acc[2][tt]), "+a"(acc[3][tt]) : : "memory");
+            else
+                asm volatile("" : "+v"(acc[0][tt]), "+v"(acc[1][tt]), "+v"(acc[2][tt]), "+v"(acc[3][tt]) : : "memory");
+        }
+    }
+    st_load_a(c, min(kt + 3, c.KT - 1), w[R]);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <bool kFull, int W, int NT>
+__device__ __forceinline__ void st_steps(const StCtx<W, NT>& c, u4v* lds, StWeights (&w)[3], StFill<W, NT>& f,
+                                         v4f (&acc)[4][NT]) {
+    const int KT = c.KT;
+    int kt = 0;
+#pragma unroll 1
+    for (; kt + 3 <= KT; kt += 3) {
+        st_step<0, kFull>(c, lds, kt, w, f, acc);
+        st_step<1, kFull>(c, lds, kt + 1, w, f, acc);
+        st_step<2, kFull>(c, lds, kt + 2, w, f, acc);
+    }
+    const int rem = KT - kt;   // block-uniform
+    if (rem > 0) st_step<0, kFull>(c, lds, kt, w, f, acc);
+    if (rem > 1) st_step<1, kFull>(c, lds, kt + 1, w, f, acc);
+}
+
+template <int W, int NT>
+__device__ __forceinline__ void st_mainloop(const StCtx<W, NT>& c, u4v* lds, v4f (&acc)[4][NT]) {
+    const int KT = c.KT;
+    StWeights w[3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q) st_load_a(c, min(q, KT - 1), w[q]);
+    StFill<W, NT> f;
+    st_load(c, 0, f);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int tt = 0; tt < NT; ++tt) acc[t][tt] = (v4f){0.f, 0.f, 0.f, 0.f};
+    st_store(c, lds, f);
+    st_load(c, min(1, KT - 1), f);
+    st_steps<false>(c, lds, w, f, acc);
+}
+
+template <int W, int NT>
+__global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void gate_up_stream_kernel(
+    MfmaArgs a, int groups, const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs,
+    const int32_t* __restrict__ gather_src, uint8_t* __restrict__ act_q, uint8_t* __restrict__ act_s) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int u, ig, ne;
+    if (!unit_block_work(a, groups, u, ig, ne)) return;
+    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    if (!unit_ok(a, e, row0, nrows)) return;
+    const bool shared = e == a.n_experts;
+    const int inter = shared ? a.shared_inter : a.inter;
+    const int items = inter / 32, item0 = ig * W;
+    if (item0 >= items) return;
+    const int H = a.hidden, nk = a.n * a.topk, topk = a.topk, n = a.n;
+    const int spitch = scale_pitch(H);
+    auto token = [&](int col) -> int {
+        const int gr = row0 + col;
+        if (shared) return gr - nk;
+        const int i = gather_src[gr];
+        const int tk = (i < 0 || i >= nk) ? 0 : i / topk;
+        return tk < n ? tk : 0;
+    };
+    StCtx<W, NT> c;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int item = item0 + wave;
+    st_context(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
+               shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), H / 128, nrows, xq,
+               (size_t)n * H, xs, (size_t)n * spitch, [&](int col) { return (uint32_t)token(col) * (uint32_t)H; },
+               [&](int col) { return (uint32_t)token(col) * (uint32_t)spitch; });
+    v4f acc[4][NT];
+    st_mainloop(c, reinterpret_cast<u4v*>(lds_raw), acc);
+    if (item >= items) return;
+
+    // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
+    const int cc = c.lane & 15, g = c.lane >> 4;
+    const int apitch = scale_pitch(a.act_ld);
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+        if (tt >= c.ntile) continue;
+        const int col = tt * 16 + cc;
+        float r0[4], r1[4];
+        float amax = 0.0f;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            r0[v] = swiglu_fast(acc[0][tt][v], acc[2][tt][v], a.limit);
+            r1[v] = swiglu_fast(acc[1][tt][v], acc[3][tt][v], a.limit);
+            amax = fmaxf(amax, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        if (col < nrows) {
+            const uint32_t sb = block_scale_e8m0(amax);
+            const float inv = u2f((254u - sb) << 23);
+            const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
+            const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
+            uint8_t* dst = act_q + (size_t)(row0 + col) * a.act_ld + (size_t)item * 32 + g * 4;
+            *reinterpret_cast<uint32_t*>(dst) = p0;
+            *reinterpret_cast<uint32_t*>(dst + 16) = p1;
+            if (g == 0) act_s[(size_t)(row0 + col) * apitch + scale_pos(item)] = (uint8_t)sb;
+        }
+    }
+}
+
+template <int W, int NT, typename YT>
+__global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void down_stream_kernel(MfmaArgs a, int groups,
+                                                                                   const uint8_t* __restrict__ act_q,
+                                                                                   const uint8_t* __restrict__ act_s,
+                                                                                   YT* __restrict__ y) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    int u, ig, ne;
+    if (!unit_block_work(a, groups, u, ig, ne)) return;
+    const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
+    if (!unit_ok(a, e, row0, nrows)) return;
+    const bool shared = e == a.n_experts;
+    const int inter = shared ? a.shared_inter : a.inter;
+    const int H = a.hidden, items = H / 64, item0 = ig * W;
+    if (item0 >= items) return;
+    const int apitch = scale_pitch(a.act_ld), act_ld = a.act_ld;
+    StCtx<W, NT> c;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int item = item0 + wave;
+    st_context(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
+               shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), inter / 128, nrows,
+               act_q + (size_t)row0 * act_ld, (size_t)nrows * act_ld, act_s + (size_t)row0 * apitch, (size_t)nrows * apitch,
+               [&](int col) { return (uint32_t)col * (uint32_t)act_ld; },
+               [&](int col) { return (uint32_t)col * (uint32_t)apitch; });
+    v4f acc[4][NT];
+    st_mainloop(c, reinterpret_cast<u4v*>(lds_raw), acc);
+    if (item >= items) return;
+
+    const int cc = c.lane & 15, g = c.lane >> 4;
+#pragma unroll
+    for (int tt = 0; tt < NT; ++tt) {
+        if (tt >= c.ntile) continue;
+        const int col = tt * 16 + cc;
+        if (col < nrows) {
+            YT* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const v4f r = acc[t][tt];
+                if constexpr (sizeof(YT) == 4)
+                    *reinterpret_cast<float4*>(dst + t * 16) = make_float4(r[0], r[1], r[2], r[3]);
+                else
+                    *reinterpret_cast<uint2*>(dst + t * 16) =
+                        make_uint2(bf16_rne(r[0]) | (bf16_rne(r[1]) << 16), bf16_rne(r[2]) | (bf16_rne(r[3]) << 16));
+            }
+        }
+    }
+}
+
 // ---- launchers ----------------------------------------------------------------------------------------
 constexpr int GU_WAVES = 4;
 constexpr int GU_WAVES_RESIDENT_X2 = 8;
@@ -826,6 +1205,10 @@ static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int
     a.limit = s.swiglu_limit;
     a.unit_cap = units.unit_rows_cap;
     a.max_units = units.max_units;
+    a.n_early = units.n_early;
+    a.dense_row0 = units.dense_row0;
+    // the gate/up launch behind the routing kernel leaves out what was computed ahead; down covers every unit
+    a.unit_range = (!down && units.n_early > 0) ? units.unit_range : nullptr;
     return a;
 }
 
@@ -837,8 +1220,30 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     const int imax = a.act_ld;
     const bool x2 = xin.q2 != nullptr;
     if (x2 != (act.q2 != nullptr)) return FERRITE_ERR_INVALID_ARG;
-    if (units.unit_rows_cap == PF_ROWS) {
+    if (units.unit_rows_cap >= PF_ROWS) {
         if (x2) return FERRITE_ERR_INVALID_ARG;   // the 128-row kernels take one-term activations
+        const int variant = g_prefill_variant.load(std::memory_order_relaxed);
+        if (variant != 0 || units.unit_rows_cap != PF_ROWS) {
+            auto go = [&](auto kernel, int W, size_t lds) -> int {
+                const int groups = (imax / 32 + W - 1) / W;
+                const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+                hipExtLaunchKernelGGL(kernel, dim3(blocks), dim3(W * 64), (uint32_t)lds, st, k_start, k_stop, 0, a, groups,
+                                      xin.q, xin.s, gather_src, act.q, act.s);
+                return check_launch("gate_up_stream");
+            };
+            int rc;
+            if (units.unit_rows_cap == 256) {
+                if ((rc = LdsLimit<&gate_up_stream_kernel<4, 16>>::ensure(StCfg<4, 16>::LDS_BYTES))) return rc;
+                return go(gate_up_stream_kernel<4, 16>, 4, StCfg<4, 16>::LDS_BYTES);
+            }
+            if (units.unit_rows_cap != PF_ROWS) return FERRITE_ERR_INVALID_ARG;
+            if (variant == 2) {
+                if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
+                return go(gate_up_stream_kernel<8, 8>, 8, StCfg<8, 8>::LDS_BYTES);
+            }
+            if ((rc = LdsLimit<&gate_up_stream_kernel<4, 8>>::ensure(StCfg<4, 8>::LDS_BYTES))) return rc;
+            return go(gate_up_stream_kernel<4, 8>, 4, StCfg<4, 8>::LDS_BYTES);
+        }
         const int groups = (imax / 32 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
         int rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES);
@@ -883,12 +1288,63 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     return check_launch("gate_up_mfma");
 }
 
+// The routing-independent part of gate/up (gate_up_early_kernel): needs the quantised x and nothing else.
+int launch_gate_up_early(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& xin, int n,
+                         const UnitTables& units, const ActPlanes& act, hipStream_t st) {
+    if (units.unit_rows_cap != 16 || units.n_early <= 0) return FERRITE_ERR_INVALID_ARG;
+    MfmaArgs a = make_args(s, packed, n, units, false);
+    a.unit_range = nullptr;
+    const bool x2 = xin.q2 != nullptr;
+    if (x2 != (act.q2 != nullptr)) return FERRITE_ERR_INVALID_ARG;
+    const int KT = s.hidden / 128, imax = a.act_ld;
+    const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
+    const size_t work = (size_t)(units.n_early + (s.shared_inter > 0 ? 1 : 0)) * ((n + 15) / 16) * groups;
+    const unsigned blocks = (unsigned)((work + 7) / 8 * 8);
+    int rc;
+    if (x2) {
+        const size_t lds = b_lds_bytes<true, kWindowKt>(KT);
+        if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, true, kWindowKt>>::ensure(lds))) return rc;
+        gate_up_early_kernel<GU_WAVES, true, kWindowKt><<<blocks, GU_WAVES * 64, lds, st>>>(a, groups, xin, act);
+    } else {
+        const size_t lds = b_lds_bytes<false, 0>(KT);
+        if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, false, 0>>::ensure(lds))) return rc;
+        gate_up_early_kernel<GU_WAVES, false, 0><<<blocks, GU_WAVES * 64, lds, st>>>(a, groups, xin, act);
+    }
+    return check_launch("gate_up_early");
+}
+
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& act, int n,
-                     const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
+                     const int32_t* gather_src, const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
     MfmaArgs a = make_args(s, packed, n, units, true);
     const bool x2 = act.q2 != nullptr;
-    if (units.unit_rows_cap == PF_ROWS) {
+    if (units.unit_rows_cap >= PF_ROWS) {
         if (x2) return FERRITE_ERR_INVALID_ARG;
+        const int variant = g_prefill_variant.load(std::memory_order_relaxed);
+        if (variant != 0 || units.unit_rows_cap != PF_ROWS) {
+            auto go = [&](auto kernel, int W, size_t lds, auto* yp) -> int {
+                const int groups = (s.hidden / 64 + W - 1) / W;
+                const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+                kernel<<<blocks, W * 64, lds, st>>>(a, groups, act.q, act.s, yp);
+                return check_launch("down_stream");
+            };
+            int rc;
+            const bool bf = y_dtype == FERRITE_DT_BF16;
+            uint16_t* yh = static_cast<uint16_t*>(y);
+            float* yf = static_cast<float*>(y);
+            if (units.unit_rows_cap == 256) {
+                constexpr size_t lds = StCfg<4, 16>::LDS_BYTES;
+                if ((rc = LdsLimit<&down_stream_kernel<4, 16, uint16_t>>::ensure(lds))) return rc;
+                if ((rc = LdsLimit<&down_stream_kernel<4, 16, float>>::ensure(lds))) return rc;
+                return bf ? go(down_stream_kernel<4, 16, uint16_t>, 4, lds, yh) : go(down_stream_kernel<4, 16, float>, 4, lds, yf);
+            }
+            if (units.unit_rows_cap != PF_ROWS) return FERRITE_ERR_INVALID_ARG;
+            if (variant == 2) {
+                constexpr size_t lds = StCfg<8, 8>::LDS_BYTES;
+                return bf ? go(down_stream_kernel<8, 8, uint16_t>, 8, lds, yh) : go(down_stream_kernel<8, 8, float>, 8, lds, yf);
+            }
+            constexpr size_t lds = StCfg<4, 8>::LDS_BYTES;
+            return bf ? go(down_stream_kernel<4, 8, uint16_t>, 4, lds, yh) : go(down_stream_kernel<4, 8, float>, 4, lds, yf);
+        }
         const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
         int rc;
@@ -901,7 +1357,7 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
         }
         return check_launch("down_prefill");
     }
-    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
+    if (units.unit_rows_cap != 16 || (units.n_early > 0 && !gather_src)) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = x2 ? b_lds_bytes<true, kWindowKt>(a.act_ld / 128) : b_lds_bytes<false, 0>(a.act_ld / 128);
     const int items = s.hidden / 64;
     const int groups = (items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW);
@@ -910,10 +1366,10 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
     int rc;
     if (x2) {
         if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(lds))) return rc;
-        down_mfma_kernel<DN_WAVES, DN_IPW, true><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, static_cast<float*>(y));
+        down_mfma_kernel<DN_WAVES, DN_IPW, true><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, gather_src, static_cast<float*>(y));
     } else {
         if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(lds))) return rc;
-        down_mfma_kernel<DN_WAVES, DN_IPW, false><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, static_cast<float*>(y));
+        down_mfma_kernel<DN_WAVES, DN_IPW, false><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, gather_src, static_cast<float*>(y));
     }
     return check_launch("down_mfma");
 }
@@ -923,6 +1379,8 @@ int warmup_experts_mfma() {
     if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false, 0>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true, kWindowKt>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES_RESIDENT_X2, true, 0>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, false, 0>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, true, kWindowKt>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES))) return rc;
