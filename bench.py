@@ -33,8 +33,14 @@ MFMA_PEAK_FP4_TFLOPS = 10100.0 # dense MXFP4 x MXFP4
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
 # counters' reading for a 1 GiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw values
-# are in profiles/.  Counters cannot be read inside this script.
-MEASURED_TRAFFIC = {("c1", "gate_up_mfma_kernel"): 764.6e6, ("c2", "gate_up_prefill_kernel"): 1470.3e6}
+# are in profiles/.  Counters cannot be read inside this script, so each figure carries the build id of the
+# library it was measured on: a run on another build reports traffic null and names the profiled build.
+MEASURED_TRAFFIC = {}   # (config, kernel) -> (bytes per launch, build id); filled in from profiles/ below
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "measured_traffic.json")
+if os.path.exists(TRAFFIC_FILE):
+    with open(TRAFFIC_FILE) as _f:
+        for _e in json.load(_f)["entries"]:
+            MEASURED_TRAFFIC[(_e["config"], _e["kernel"])] = (_e["bytes_per_launch"], _e["build_id"])
 
 WORKLOADS = {
     "c0": "c0: tiny parity layer, 8 tokens, H256 E16 top4 (4 groups/2) I128, MXFP4 weights, f32 activations",
@@ -121,21 +127,127 @@ def stage_profile(hip, ev, layer, x, out, mode, ws, reps):
     return stage_us, eager_us, gu_kernel_us
 
 
-def gate_up_roofline(cfg, n, unit_rows, gu_us, ab, traffic_key):
+def measured_traffic(config, kernel, build_id):
+    """{"traffic": bytes or None[, "traffic_stale_build": id]} for the roofline object."""
+    hit = MEASURED_TRAFFIC.get((config, kernel))
+    if hit is None:
+        return {"traffic": None}
+    if hit[1] != build_id:
+        return {"traffic": None, "traffic_stale_build": hit[1], "traffic_of_that_build": hit[0]}
+    return {"traffic": hit[0]}
+
+
+def gate_up_roofline(cfg, n, unit_rows, gu_us, ab, config_name, build_id):
     if unit_rows != 128:
         # decode-sized batch: every weight byte is streamed once per unit; the kernel is HBM bound
         gbs = ab["gate_up"] / (gu_us * 1e-6) / 1e9
-        return {"bound": "hbm", "kernel": "gate_up_mfma_kernel", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(traffic_key),
-                "algorithmic_bytes_per_launch": ab["gate_up"], "avg_launch_us": round(gu_us, 2)}
-    # prefill-sized batch: 128-row units, both operands tiled through LDS; the kernel is MFMA bound.  The MFMA takes
-    # e2m1 weights and e4m3 activations, which issues at the fp8 rate: priced against the fp8 peak
+        r = {"bound": "hbm", "kernel": "gate_up_mfma_kernel", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+             "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}
+        r.update(measured_traffic(config_name, r["kernel"], build_id))
+        r.update({"algorithmic_bytes_per_launch": ab["gate_up"], "avg_launch_us": round(gu_us, 2)})
+        return r
+    # prefill-sized batch: 128-row units; the kernel is MFMA bound.  The MFMA takes e2m1 weights and e4m3
+    # activations, which issues at the fp8 rate: priced against the fp8 peak
     gu_flops = 2.0 * n * (cfg.topk * cfg.inter + cfg.shared_inter) * 2 * cfg.hidden
     tf = gu_flops / (gu_us * 1e-6) / 1e12
-    return {"bound": "mfma", "kernel": "gate_up_prefill_kernel", "achieved": round(tf, 1), "peak": MFMA_PEAK_FP8_TFLOPS,
-            "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_FP8_TFLOPS, 4), "traffic": MEASURED_TRAFFIC.get(traffic_key),
-            "algorithmic_flops_per_launch": gu_flops, "avg_launch_us": round(gu_us, 2),
-            "frac_of_fp4_peak": round(tf / MFMA_PEAK_FP4_TFLOPS, 4)}
+    r = {"bound": "mfma", "kernel": "gate_up_stream_kernel", "achieved": round(tf, 1), "peak": MFMA_PEAK_FP8_TFLOPS,
+         "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_FP8_TFLOPS, 4)}
+    r.update(measured_traffic(config_name, r["kernel"], build_id))
+    r.update({"algorithmic_flops_per_launch": gu_flops, "avg_launch_us": round(gu_us, 2),
+              "frac_of_fp4_peak": round(tf / MFMA_PEAK_FP4_TFLOPS, 4)})
+    return r
+
+
+def f32_parity(oracle, inp, gpu_rows, ids_gpu, sel, n_threads):
+    """Distance of the GPU output rows `sel` from the f32 oracle (CpuBackend's arithmetic) on the same inputs."""
+    ref = oracle.moe_ffn_mxfp4(inp, act_mode=0, n_threads=n_threads, tok_sel=sel)
+    d = float(np.abs(gpu_rows.astype(np.float64) - ref["out"]).max() / np.abs(ref["out"]).max())
+    return {"max_abs_rel": float(f"{d:.3e}"), "tokens": int(len(sel)),
+            "router_ids_equal": bool(np.array_equal(ids_gpu, ref["ids"].astype(np.int32)))}
+
+
+def decode_step(hip, torch, synth, cfg, n_layers, mode, steps, warmup):
+    """The 42-layer decode step (configs[4]): every layer has its own weights, li_0 = x, li_{l+1} = ffn_out_l, every
+    layer normalises its input first (rmsnorm -> layer, exec/lib.rs:487-490), one workspace, ONE hipGraph per step."""
+    n = cfg.n
+    t0 = time.time()
+    layers = []
+    for li in range(n_layers):
+        inp = synth.make_inputs(cfg, seed=0, layer=li)
+        layers.append(hip.load_moe_layer(inp, keep_checkpoint_layout=False))
+        if li == 0:
+            x_in = torch.from_numpy(synth.round_to_bf16(inp.x) if cfg.act_bf16 else inp.x).to(hip.device).float().contiguous()
+        del inp
+    setup_s = time.time() - t0
+    mode = hip.effective_mode(layers[0], n, mode)
+    g = torch.Generator(device="cpu").manual_seed(2)
+    norm_ws = [(torch.rand(cfg.hidden, generator=g) + 0.5).to(hip.device) for _ in layers]
+    ping = [torch.empty(n, cfg.hidden, device=hip.device) for _ in range(2)]
+    bws = hip.block_workspace(layers[0], n, mode)
+
+    def step():
+        src = x_in
+        for i, ly in enumerate(layers):
+            dst = ping[i & 1]
+            hip.moe_block_mxfp4(ly, src, norm_ws[i], 1e-6, None, None, None, dst, mode, workspace=bws)
+            src = dst
+
+    step()
+    hip.sync()
+    hip.begin_capture()
+    step()
+    trace = hip.end_capture()
+    ms = time_replays(hip, torch, lambda: hip.begin_verify(trace), steps, warmup) * 1e3
+    hip.graph_destroy(trace)
+    # experts hit in every layer of the chain, from the tables each layer leaves in the shared workspace
+    step_bytes, src, hit = 0, x_in, []
+    for i, ly in enumerate(layers):
+        dst = ping[i & 1]
+        hip.moe_block_mxfp4(ly, src, norm_ws[i], 1e-6, None, None, None, dst, mode, workspace=bws)
+        hip.sync()
+        c = hip.workspace_view(ly, n, mode, workspace=bws)["counts"].cpu().numpy()
+        hit.append(int((c > 0).sum()))
+        step_bytes += algorithmic_bytes(cfg, n, hit[-1])["total"]
+        src = dst
+    finite = bool(torch.isfinite(ping[(n_layers - 1) & 1]).all().item())
+    return {"workload": WORKLOADS["c4"], "tokens": n, "layers": n_layers, "steps": steps,
+            "activation_terms": {1: "fp8", 2: "fp8x2"}[mode],
+            "ms_per_step": round(ms, 4), "us_per_layer": round(ms * 1e3 / n_layers, 2),
+            "tokens_per_s": round(n / (ms * 1e-3), 1), "step_algorithmic_bytes": step_bytes,
+            "step_hbm_gbs": round(step_bytes / (ms * 1e-3) / 1e9, 1),
+            "step_hbm_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "experts_hit_min": min(hit), "output_finite": finite, "setup_s": round(setup_s, 1)}, layers, step_bytes
+
+
+def layer_leg(hip, torch, ev, layer, x, n, cfg, mode, steps, warmup, stack=True):
+    """One layer per captured graph: seconds-per-replay timing, the same layer eight times inside one graph, the
+    per-stage events and the gate/up kernel's own duration."""
+    from ferrite_amd.backend import MODE_MFMA_FP8_X2
+    out = torch.empty(n, cfg.hidden, dtype=x.dtype, device=hip.device)
+    ws = hip.workspace(layer, n, mode)
+    for _ in range(3):
+        hip.moe_layer_dev_mxfp4(layer, x, out, mode, ws)
+    hip.sync()
+    hip.begin_capture()
+    hip.moe_layer_dev_mxfp4(layer, x, out, mode, ws)
+    trace = hip.end_capture()
+    us = time_replays(hip, torch, lambda: hip.begin_verify(trace), steps, warmup) * 1e6
+    hip.graph_destroy(trace)
+    us_stack = None
+    if stack:
+        STACK = 8
+        hip.begin_capture()
+        for _ in range(STACK):
+            hip.moe_layer_dev_mxfp4(layer, x, out, mode, ws)
+        st = hip.end_capture()
+        us_stack = time_replays(hip, torch, lambda: hip.begin_verify(st), max(4, min(50, steps // 4)), 3) / STACK * 1e6
+        hip.graph_destroy(st)
+    stage_us, eager_us, gu_us = stage_profile(hip, ev, layer, x, out, mode, ws, min(steps, 50))
+    gpu_out = out.float().cpu().numpy()
+    view = hip.workspace_view(layer, n, mode)
+    return dict(us=us, us_stack=us_stack, stage_us=stage_us, eager_us=eager_us, gu_us=gu_us, out=gpu_out,
+                ids=view["ids"].cpu().numpy(), counts=view["counts"].cpu().numpy(),
+                terms="fp8x2" if mode == MODE_MFMA_FP8_X2 else "fp8")
 
 
 def main():
@@ -148,12 +260,14 @@ def main():
     ap.add_argument("--layers", type=int, default=0,
                     help="chain this many distinct layers into one captured step (default: 42 for c4, else 1)")
     ap.add_argument("--mode", default="auto", choices=["auto", "fp8", "fp8x2"],
-                    help="activation format of the expert GEMMs: one e4m3 term, two (decode-sized batches only), or "
-                         "auto = two where they are supported")
+                    help="activation format of the expert GEMMs: one e4m3 term, two (decode-sized batches; larger ones "
+                         "fall back to one), or auto = two where the library takes them")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-load-bench", action="store_true",
                     help="skip the checkpoint -> packed-buffer load measurement (writes a shard of the layer to TMPDIR)")
     ap.add_argument("--no-prefill-leg", action="store_true", help="skip the 4096-token leg of the default run")
+    ap.add_argument("--no-decode-step-leg", action="store_true",
+                    help="skip the 42-layer decode step (54 GB of weights, about a minute of set-up) of the default run")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of graph replays")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run a plain device copy of this many MiB (a counter calibration point for rocprofv3 --pmc)")
@@ -171,48 +285,12 @@ def main():
         cfg = cfg.with_tokens(args.tokens)
     n = cfg.n
     hip = HipBackend()
+    ev = HipEvents()
     n_layers = args.layers or (42 if args.config == "c4" else 1)
-    decode_sized = n * cfg.topk < 48 * cfg.n_experts
-    if args.mode == "fp8x2" and not decode_sized:
-        print("--mode fp8x2 is for decode-sized batches (n*topk < 48*experts)", file=sys.stderr)
-        sys.exit(2)
-    mode = MODE_MFMA_FP8_X2 if (args.mode == "fp8x2" or (args.mode == "auto" and decode_sized)) else MODE_MFMA_FP8
-    mode_name = {MODE_MFMA_FP8: "fp8", MODE_MFMA_FP8_X2: "fp8x2"}[mode]
-    t0 = time.time()
-    inp = synth.make_inputs(cfg, seed=0)
-    layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
-    layers = [layer]
-    for li in range(1, n_layers):
-        extra = synth.make_inputs(cfg, seed=0, layer=li)
-        layers.append(hip.load_moe_layer(extra, keep_checkpoint_layout=False))
-        del extra
-    t_setup = time.time() - t0
-
-    x = torch.from_numpy(inp.x).to(hip.device)
-    if cfg.act_bf16:
-        x = x.to(torch.bfloat16)
-    out = torch.empty(n, cfg.hidden, dtype=x.dtype, device=hip.device)
-    ws = hip.workspace(layer, n, mode)
-
-    if n_layers == 1:
-        def step():
-            hip.moe_layer_dev_mxfp4(layer, x, out, mode, ws)
-    else:
-        # The chained step: li_0 = x; li_{l+1} = ffn_out_l; every layer normalises its input first (rmsnorm ->
-        # layer, exec/lib.rs:487-490), which keeps the activations, and with them the routing, at their scale through
-        # all layers.  One workspace; the input buffer is never written, so replays start from the same data.
-        g = torch.Generator(device="cpu").manual_seed(2)
-        norm_ws = [(torch.rand(cfg.hidden, generator=g) + 0.5).to(hip.device) for _ in layers]
-        x_in = x.float().contiguous()
-        ping = [torch.empty(n, cfg.hidden, device=hip.device) for _ in range(2)]
-        bws = hip.block_workspace(layer, n, mode)
-
-        def step():
-            src = x_in
-            for i, ly in enumerate(layers):
-                dst = ping[i & 1]
-                hip.moe_block_mxfp4(ly, src, norm_ws[i], 1e-6, None, None, None, dst, mode, workspace=bws)
-                src = dst
+    asked = MODE_MFMA_FP8 if args.mode == "fp8" else MODE_MFMA_FP8_X2   # auto: two terms where they are taken
+    oracle = None
+    if not args.no_cpu_baseline:
+        from oracle import binding as oracle
 
     if args.calib_copy_mib:
         src = torch.ones(args.calib_copy_mib << 20, dtype=torch.uint8, device=hip.device)
@@ -222,36 +300,86 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # warm up eagerly (fills caches), then capture one step as a graph
-    for _ in range(max(min(args.warmup, 5), 2)):
-        step()
-    hip.sync()
-    trace = None
-    if not args.no_graph:
-        hip.begin_capture()
-        step()
-        trace = hip.end_capture()
-    replay = step if trace is None else (lambda: hip.begin_verify(trace))
-    ms_per_step = time_replays(hip, torch, replay, args.steps, args.warmup) * 1e3
+    # ---- the chained decode step (configs[4]) as the workload of its own ----
+    if n_layers > 1:
+        step, layers, step_bytes = decode_step(hip, torch, synth, cfg, n_layers, asked, args.steps, args.warmup)
+        mode = hip.effective_mode(layers[0], n, asked)
+        inp = synth.make_inputs(cfg, seed=0)
+        x = torch.from_numpy(inp.x).to(hip.device)
+        x = x.to(torch.bfloat16) if cfg.act_bf16 else x
+        leg = layer_leg(hip, torch, ev, layers[0], x, n, cfg, mode, min(args.steps, 50), 3, stack=False)
+        n_active = int((leg["counts"] > 0).sum())
+        ab = algorithmic_bytes(cfg, n, n_active)
+        unit_rows = hip.unit_rows(layers[0], n, mode)
+        ms = step["ms_per_step"]
+        result = {
+            "metric": "moe_layer_tokens_per_s", "value": round(n * n_layers / (ms * 1e-3), 1), "unit": "tokens/s",
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "mxfp4 x e4m3 (two terms) -> f32" if mode == MODE_MFMA_FP8_X2 else "mxfp4 x e4m3 -> f32",
+            "data": "synthetic",
+            "config": {"workload": WORKLOADS[args.config], "tokens": n, "hidden": cfg.hidden, "experts": cfg.n_experts,
+                       "topk": cfg.topk, "n_group": cfg.n_group, "topk_group": cfg.topk_group, "inter": cfg.inter,
+                       "activation_terms": leg["terms"], "launch": "hipGraph replay", "layers": n_layers,
+                       "value_counts": "token-layers per second (tokens x layers / step time)"},
+            "layers_per_step": n_layers, "step_algorithmic_bytes": step_bytes, "step_hbm_gbs": step["step_hbm_gbs"],
+            "step_hbm_frac": step["step_hbm_frac"], "us_per_layer": step["us_per_layer"],
+            "stage_us_one_layer": {k: round(v, 2) for k, v in leg["stage_us"].items()},
+            "experts_hit": n_active, "unit_rows": unit_rows, "output_finite": step["output_finite"],
+            "roofline": gate_up_roofline(cfg, n, unit_rows, leg["gu_us"], ab, None if args.tokens else args.config,
+                                         hip.build_id),
+            "cpu_baseline": None, "setup_s": step["setup_s"], "build_id": hip.build_id,
+        }
+        print(json.dumps(result))
+        return
 
-    # A graph launch costs about 13 us on the device before its first kernel starts; a model runs all its layers
-    # from one graph, so the same layer is also timed eight times back to back inside one graph (reported as
-    # us_per_layer_in_stack; `value` stays the single-layer-per-launch figure).
-    us_in_stack = None
-    if trace is not None and n_layers == 1:
-        STACK = 8
-        hip.begin_capture()
-        for _ in range(STACK):
-            step()
-        stack_trace = hip.end_capture()
-        reps = max(4, min(50, args.steps // 4))
-        us_in_stack = time_replays(hip, torch, lambda: hip.begin_verify(stack_trace), reps, 3) / STACK * 1e6
-        hip.graph_destroy(stack_trace)
+    t0 = time.time()
+    inp = synth.make_inputs(cfg, seed=0)
+    layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
+    t_setup = time.time() - t0
+    mode = hip.effective_mode(layer, n, asked)   # the library declines two terms for prefill-sized batches
+    x = torch.from_numpy(inp.x).to(hip.device)
+    if cfg.act_bf16:
+        x = x.to(torch.bfloat16)
 
-    # The FFN half of a decoder layer around the same layer (exec/lib.rs:487-492): rmsnorm -> layer -> hc_post as one
-    # captured call, and the two neighbours on their own (torch events on the backend's stream).
+    if args.no_graph:
+        out = torch.empty(n, cfg.hidden, dtype=x.dtype, device=hip.device)
+        ws = hip.workspace(layer, n, mode)
+        us = time_replays(hip, torch, lambda: hip.moe_layer_dev_mxfp4(layer, x, out, mode, ws), args.steps, args.warmup) * 1e6
+        stage_us, eager_us, gu_us = stage_profile(hip, ev, layer, x, out, mode, ws, min(args.steps, 50))
+        view = hip.workspace_view(layer, n, mode)
+        leg = dict(us=us, us_stack=None, stage_us=stage_us, eager_us=eager_us, gu_us=gu_us, out=out.float().cpu().numpy(),
+                   ids=view["ids"].cpu().numpy(), counts=view["counts"].cpu().numpy(),
+                   terms="fp8x2" if mode == MODE_MFMA_FP8_X2 else "fp8")
+    else:
+        leg = layer_leg(hip, torch, ev, layer, x, n, cfg, mode, args.steps, args.warmup)
+    ms_per_step = leg["us"] * 1e-3
+    counts = leg["counts"]
+    n_active = int((counts > 0).sum())
+    ab = algorithmic_bytes(cfg, n, n_active)
+    flops = 2.0 * n * (cfg.topk * cfg.inter + cfg.shared_inter) * 3 * cfg.hidden
+    unit_rows = hip.unit_rows(layer, n, mode)
+    roofline = gate_up_roofline(cfg, n, unit_rows, leg["gu_us"], ab, None if args.tokens else args.config, hip.build_id)
+    default_run = args.config == "c1" and not args.tokens and not args.no_graph
+    ncores = min(16, os.cpu_count() or 1)
+
+    # the reference's own serving format beside the two-term one: same layer, one e4m3 term (quant.rs:201-214)
+    decode_fp8 = None
+    if default_run and mode == MODE_MFMA_FP8_X2:
+        l1 = layer_leg(hip, torch, ev, layer, x, n, cfg, MODE_MFMA_FP8, max(20, args.steps // 2), 5)
+        decode_fp8 = {"activation_terms": "fp8", "us_per_layer": round(l1["us"], 2),
+                      "us_per_layer_in_stack": round(l1["us_stack"], 2),
+                      "gate_up_kernel_us": round(l1["gu_us"], 2),
+                      "layer_hbm_frac": round(ab["total"] / (l1["us"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                      "what": "the same layer with one e4m3 term per activation, the reference's serving format"}
+        if oracle is not None:
+            decode_fp8["parity_vs_f32_oracle"] = f32_parity(oracle, inp, l1["out"][:min(n, 32)], l1["ids"],
+                                                            np.arange(min(n, 32), dtype=np.int32), ncores)
+
+    # the FFN half of a decoder layer around the same layer (exec/lib.rs:487-492): rmsnorm -> layer -> hc_post as one
+    # captured call, and the two neighbours on their own (torch events on the backend's stream)
     block = None
-    if trace is not None and n_layers == 1:
+    if not args.no_graph:
         nh = 4
         g = torch.Generator(device="cpu").manual_seed(1)
         li = (torch.randn(n, cfg.hidden, generator=g) * 3.0).to(hip.device)
@@ -285,70 +413,47 @@ def main():
         block = {"us_per_block": round(us_block, 2), "hc_streams": nh,
                  "rmsnorm_us": round(op_us(lambda: hip.rmsnorm(li, norm_w, 1e-6, hfn)), 2),
                  "hc_post_us": round(op_us(lambda: hip.hc_post(hfn, residual, post, comb)), 2)}
+        del li, residual, bout, hfn
 
-    ev = HipEvents()
-    stage_us, eager_us, gu_kernel_us = stage_profile(hip, ev, layer, x, out, mode, ws, min(args.steps, 50))
-    gpu_out = out.float().cpu().numpy()      # layer 0 on the config's own input (the eager passes just above)
-
-    view = hip.workspace_view(layer, n, mode)
-    counts = view["counts"].cpu().numpy()
-    n_active = int((counts > 0).sum())
-    ab = algorithmic_bytes(cfg, n, n_active)
-    step_bytes = ab["total"] * n_layers
-    if n_layers > 1:
-        # experts hit in every layer of the chain, from the tables each layer leaves in the shared workspace
-        step_bytes, src = 0, x_in
-        for i, ly in enumerate(layers):
-            dst = ping[i & 1]
-            hip.moe_block_mxfp4(ly, src, norm_ws[i], 1e-6, None, None, None, dst, mode, workspace=bws)
-            hip.sync()
-            c = hip.workspace_view(ly, n, mode, workspace=bws)["counts"].cpu().numpy()
-            step_bytes += algorithmic_bytes(cfg, n, int((c > 0).sum()))["total"]
-            src = dst
-    flops = 2.0 * n * (cfg.topk * cfg.inter + cfg.shared_inter) * 3 * cfg.hidden
-
-    us_layer = ms_per_step * 1e3 / n_layers
-    unit_rows = hip.unit_rows(layer, n, mode)
-    kname = "gate_up_prefill_kernel" if unit_rows == 128 else "gate_up_mfma_kernel"
-    roofline = gate_up_roofline(cfg, n, unit_rows, gu_kernel_us, ab, None if args.tokens else (args.config, kname))
-
-    # the other half of the metric on the same weights: the 4096-token prefill chunk (c2 is c1's layer at n = 4096),
-    # one e4m3 term as that configuration prescribes; a bounded number of replays
+    # the other half of the metric on the same weights: the 4096-token prefill chunk (c2 is c1's layer at n = 4096).
+    # Asked for in the same mode as the decode leg: the library declines two terms at this size and the backend falls
+    # back to one e4m3 term, the format that configuration prescribes
     prefill = None
-    if args.config == "c1" and not args.tokens and not args.no_prefill_leg and trace is not None:
+    if default_run and not args.no_prefill_leg:
         pcfg = synth.CONFIGS["c2"]
         pn = pcfg.n
-        px = torch.from_numpy(synth.make_activations(pcfg, seed=0)).to(hip.device).to(torch.bfloat16)
-        pout = torch.empty(pn, pcfg.hidden, dtype=torch.bfloat16, device=hip.device)
-        pws = hip.workspace(layer, pn, MODE_MFMA_FP8)
-        for _ in range(3):
-            hip.moe_layer_dev_mxfp4(layer, px, pout, MODE_MFMA_FP8, pws)
-        hip.sync()
-        hip.begin_capture()
-        hip.moe_layer_dev_mxfp4(layer, px, pout, MODE_MFMA_FP8, pws)
-        ptrace = hip.end_capture()
-        p_steps = max(10, min(50, args.steps))
-        p_us = time_replays(hip, torch, lambda: hip.begin_verify(ptrace), p_steps, 5) * 1e6
-        hip.graph_destroy(ptrace)
-        p_stage, _, p_gu_us = stage_profile(hip, ev, layer, px, pout, MODE_MFMA_FP8, pws, 10)
-        pcounts = hip.workspace_view(layer, pn, MODE_MFMA_FP8)["counts"].cpu().numpy()
+        px_np = synth.make_activations(pcfg, seed=0)
+        px = torch.from_numpy(px_np).to(hip.device).to(torch.bfloat16)
+        pmode = hip.effective_mode(layer, pn, asked)
+        pl = layer_leg(hip, torch, ev, layer, px, pn, pcfg, pmode, max(10, min(50, args.steps)), 5, stack=False)
+        pcounts = pl["counts"]
         pab = algorithmic_bytes(pcfg, pn, int((pcounts > 0).sum()))
         pflops = 2.0 * pn * (pcfg.topk * pcfg.inter + pcfg.shared_inter) * 3 * pcfg.hidden
-        ptf = pflops / (p_us * 1e-6) / 1e12
-        prefill = {"workload": WORKLOADS["c2"], "tokens": pn, "steps": p_steps, "us_per_layer": round(p_us, 2),
-                   "tokens_per_s": round(pn / (p_us * 1e-6), 1), "layer_tflops": round(ptf, 1),
+        ptf = pflops / (pl["us"] * 1e-6) / 1e12
+        prefill = {"workload": WORKLOADS["c2"], "tokens": pn, "steps": max(10, min(50, args.steps)),
+                   "activation_terms": pl["terms"], "us_per_layer": round(pl["us"], 2),
+                   "tokens_per_s": round(pn / (pl["us"] * 1e-6), 1), "layer_tflops": round(ptf, 1),
                    "mfma_frac_of_fp8_peak": round(ptf / MFMA_PEAK_FP8_TFLOPS, 4),
                    "mfma_frac_of_mxfp4_peak": round(ptf / MFMA_PEAK_FP4_TFLOPS, 4),
-                   "stage_us": {k: round(v, 2) for k, v in p_stage.items()},
+                   "stage_us": {k: round(v, 2) for k, v in pl["stage_us"].items()},
                    "max_over_mean_tokens_per_expert": round(float(pcounts.max() / max(pcounts.mean(), 1e-9)), 2),
-                   "roofline": gate_up_roofline(pcfg, pn, hip.unit_rows(layer, pn, MODE_MFMA_FP8), p_gu_us, pab,
-                                                ("c2", "gate_up_prefill_kernel"))}
-        del px, pout
+                   "roofline": gate_up_roofline(pcfg, pn, hip.unit_rows(layer, pn, pmode), pl["gu_us"], pab, "c2",
+                                                hip.build_id)}
+        if oracle is not None:
+            # the same 32-token sample the CPU baseline takes: evenly spaced tokens of the chunk, routed on the CPU too
+            import dataclasses
+            sel = np.linspace(0, pn - 1, 32).astype(np.int32)
+            pinp = dataclasses.replace(inp, cfg=pcfg, x=synth.round_to_bf16(px_np))
+            prefill["parity_vs_f32_oracle"] = f32_parity(oracle, pinp, pl["out"][sel], pl["ids"], sel, ncores)
+            prefill["parity_vs_f32_oracle"]["what"] = ("one e4m3 term per activation (three mantissa bits) against the "
+                                                       "unquantised f32 oracle; router ids compared for all tokens")
+            del pinp
+        del px, pl
 
     # the row before the layer: one layer's shard (safetensors, the reference's tensor names) streamed from the
     # page cache into the packed buffer; PCIe-bound, priced against a pinned -> device copy of the same size
     load = None
-    if not args.no_load_bench and n_layers == 1:
+    if not args.no_load_bench:
         try:
             import tempfile
             from ferrite_amd import checkpoint as ckpt
@@ -386,12 +491,11 @@ def main():
             load = {"error": f"{type(e).__name__}: {e}"}
 
     cpu, parity = None, None
-    if not args.no_cpu_baseline:
-        from oracle import binding as oracle
+    if oracle is not None:
         # the whole layer for a bounded token sample, single thread (the reference's CpuBackend is
         # single-threaded scalar code), f32 activations as CpuBackend computes
         ns = min(n, 32)
-        sel = np.arange(ns, dtype=np.int32)
+        sel = np.linspace(0, n - 1, ns).astype(np.int32)
         reps = 0
         t0 = time.perf_counter()
         while True:
@@ -400,21 +504,32 @@ def main():
             if time.perf_counter() - t0 > 12.0 or reps >= 12:
                 break
         t1 = (time.perf_counter() - t0) / reps
-        ncores = min(16, os.cpu_count() or 1)
         t0 = time.perf_counter()
         oracle.moe_ffn_mxfp4(inp, act_mode=0, n_threads=ncores, tok_sel=sel)
         tall = time.perf_counter() - t0
+        extrap = "" if ns == n else (f"; the whole batch of {n} tokens would take {t1 * n / ns:.0f} s at this rate "
+                                     "(linear extrapolation, not measured)")
         cpu = {"value": round(ns / t1, 2), "unit": "tokens/s", "cores": 1, "kind": "port",
                "sample": f"full layer (routing of all {n} tokens + experts + shared + combine) for {ns} tokens, "
-                         f"{reps} repetition(s), {t1:.2f} s each, f32 activations",
+                         f"{reps} repetition(s), {t1:.2f} s each, f32 activations" + extrap,
                "all_cores": {"value": round(ns / tall, 2), "cores": ncores, "seconds": round(tall, 2)}}
         # the same run is the parity check of this process's GPU output: the f32 oracle is CpuBackend's arithmetic
-        ids_equal = bool(np.array_equal(view["ids"].cpu().numpy(), ref["ids"].astype(np.int32)))
-        d = float(np.abs(gpu_out[:ns].astype(np.float64) - ref["out"]).max() / np.abs(ref["out"]).max())
+        ids_equal = bool(np.array_equal(leg["ids"], ref["ids"].astype(np.int32)))
+        d = float(np.abs(leg["out"][sel].astype(np.float64) - ref["out"]).max() / np.abs(ref["out"]).max())
         parity = {"max_abs_rel": float(f"{d:.3e}"), "tokens": ns, "router_ids_equal": ids_equal,
                   "what": "max|gpu - oracle| / max|oracle| of the layer output over the sampled tokens, oracle = the f32 "
                           "CPU restatement of CpuBackend (act_mode 0); output rounded to bf16 where the config says so"}
 
+    # the 42-layer decode step of configs[4] (192 tokens) as one hipGraph: last, it needs 54 GB for its weights
+    dstep = None
+    if default_run and not args.no_decode_step_leg:
+        del layer
+        torch.cuda.empty_cache()
+        dstep, dlayers, _ = decode_step(hip, torch, synth, synth.CONFIGS["c4"], 42, asked,
+                                        max(5, min(50, args.steps)), 2)
+        del dlayers
+
+    us_layer = leg["us"]
     result = {
         "metric": "moe_layer_tokens_per_s", "value": round(n / (ms_per_step * 1e-3), 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
@@ -423,26 +538,28 @@ def main():
         "data": "synthetic",
         "config": {"workload": WORKLOADS[args.config], "tokens": n, "hidden": cfg.hidden, "experts": cfg.n_experts,
                    "topk": cfg.topk, "n_group": cfg.n_group, "topk_group": cfg.topk_group, "inter": cfg.inter,
-                   "activation_terms": mode_name, "launch": "eager" if trace is None else "hipGraph replay"},
-        "layers_per_step": n_layers, "step_algorithmic_bytes": step_bytes,
-        "step_hbm_gbs": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
-        "us_per_layer": round(us_layer, 2), "us_per_layer_eager_events": round(eager_us, 2),
-        "us_per_layer_in_stack": None if us_in_stack is None else round(us_in_stack, 2),
-        "stage_us": {k: round(v, 2) for k, v in stage_us.items()},
+                   "activation_terms": leg["terms"],
+                   "activation_format_note": "two e4m3 terms per activation is this build's own format (no reference "
+                                             "fixture); the reference's one-term format is timed under decode_fp8"
+                   if mode == MODE_MFMA_FP8_X2 else "one e4m3 term per activation, the reference's serving format",
+                   "launch": "eager" if args.no_graph else "hipGraph replay"},
+        "layers_per_step": 1, "step_algorithmic_bytes": ab["total"],
+        "step_hbm_gbs": round(ab["total"] / (ms_per_step * 1e-3) / 1e9, 1),
+        "us_per_layer": round(us_layer, 2), "us_per_layer_eager_events": round(leg["eager_us"], 2),
+        "us_per_layer_in_stack": None if leg["us_stack"] is None else round(leg["us_stack"], 2),
+        "stage_us": {k: round(v, 2) for k, v in leg["stage_us"].items()},
         "experts_hit": n_active, "max_tokens_per_expert": int(counts.max()),
         "max_over_mean_tokens_per_expert": round(float(counts.max() / max(counts.mean(), 1e-9)), 2),
         "layer_algorithmic_bytes": ab["total"],
-        "layer_hbm_gbs": round(step_bytes / n_layers / (us_layer * 1e-6) / 1e9, 1),
-        "layer_hbm_frac": round(step_bytes / n_layers / (us_layer * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+        "layer_hbm_gbs": round(ab["total"] / (us_layer * 1e-6) / 1e9, 1),
+        "layer_hbm_frac": round(ab["total"] / (us_layer * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
         "layer_tflops": round(flops / (us_layer * 1e-6) / 1e12, 2),
         "mfma_frac_of_fp8_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP8_TFLOPS, 4),
         "mfma_frac_of_mxfp4_peak": round(flops / (us_layer * 1e-6) / 1e12 / MFMA_PEAK_FP4_TFLOPS, 4),
-        "parity_vs_f32_oracle": parity, "prefill": prefill,
+        "parity_vs_f32_oracle": parity, "decode_fp8": decode_fp8, "prefill": prefill, "decode_step": dstep,
         "block_rmsnorm_layer_hc_post": block, "checkpoint_load": load, "unit_rows": unit_rows, "roofline": roofline,
         "cpu_baseline": cpu, "setup_s": round(t_setup, 1), "build_id": hip.build_id,
     }
-    if trace is not None:
-        hip.graph_destroy(trace)
     print(json.dumps(result))
 
 

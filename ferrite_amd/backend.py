@@ -29,7 +29,7 @@ ABI_VERSION = 3
 OK, ERR_INVALID_ARG, DECLINED, ERR_WORKSPACE, ERR_RUNTIME = 0, 1, 2, 3, 4
 DT_F32, DT_BF16 = 0, 1
 MODE_F32_CHECK, MODE_MFMA_FP8, MODE_MFMA_FP8_X2 = 0, 1, 2
-OVERRIDE_UNIT_ROWS, OVERRIDE_Y_F32, OVERRIDE_PREFILL_TILE, OVERRIDE_EARLY_EXPERTS = 0, 1, 2, 3
+OVERRIDE_UNIT_ROWS, OVERRIDE_Y_F32, OVERRIDE_PREFILL_TILE, OVERRIDE_EARLY_EXPERTS, OVERRIDE_HEAD = 0, 1, 2, 3, 4
 
 
 class FerriteError(RuntimeError):
@@ -90,7 +90,7 @@ EXPORTS = [
     "ferrite_moe_pack_weights", "ferrite_moe_pack_expert", "ferrite_moe_pack_router",
     "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_block_workspace_bytes", "ferrite_moe_block_mxfp4", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
     "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_static", "ferrite_moe_layer_mxfp4_timed",
-    "ferrite_moe_layer_mxfp4_ov", "ferrite_overlap_create", "ferrite_overlap_destroy", "ferrite_moe_layer_early_experts",
+    "ferrite_moe_layer_check", "ferrite_moe_layer_mxfp4_ov", "ferrite_overlap_create", "ferrite_overlap_destroy", "ferrite_moe_layer_early_experts",
     "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
     "ferrite_graph_destroy",
 ]
@@ -142,6 +142,7 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_overlap_create.argtypes = [C.POINTER(vp)]
     lib.ferrite_overlap_destroy.argtypes = [vp]
     lib.ferrite_moe_layer_early_experts.argtypes = [C.POINTER(MoeShape), i32, i32]
+    lib.ferrite_moe_layer_check.argtypes = [C.POINTER(MoeShape), i32, i32]
     lib.ferrite_moe_layer_mxfp4_static.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp, i32, i32, vp, i32,
                                                    i32, vp]
     lib.ferrite_graph_begin.argtypes = [vp]
@@ -245,7 +246,7 @@ class HipBackend:
         self._capturing = False
         self._graphs: Dict[str, int] = {}
         self._verify_ok = False
-        self._overrides = {OVERRIDE_UNIT_ROWS: 0, OVERRIDE_Y_F32: 0, OVERRIDE_PREFILL_TILE: 0, OVERRIDE_EARLY_EXPERTS: 0}
+        self._overrides = {OVERRIDE_UNIT_ROWS: 0, OVERRIDE_Y_F32: 0, OVERRIDE_PREFILL_TILE: 0, OVERRIDE_EARLY_EXPERTS: 0, OVERRIDE_HEAD: 0}
         self._ck(self.lib.ferrite_hip_warmup(), "warmup")   # LDS limits, before any capture (cuda.rs:627-657)
         ov = C.c_void_p()
         self._ck(self.lib.ferrite_overlap_create(C.byref(ov)), "overlap_create")   # the second stream + fork/join events
@@ -529,7 +530,18 @@ class HipBackend:
         self._leave()
         return out
 
+    def effective_mode(self, layer: MoeLayer, n: int, mode: int) -> int:
+        """The mode a layer call for n tokens runs in: the one asked for, or, where the library declines it, the mode
+        the caller falls back to (cuda.rs:5763-5765: a declined fused kernel is not an error, the other path runs).
+        Two-term activations are declined for prefill-sized batches: those run with one term."""
+        rc = self.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, mode)
+        if rc == DECLINED and mode == MODE_MFMA_FP8_X2 and \
+                self.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, MODE_MFMA_FP8) == OK:
+            return MODE_MFMA_FP8
+        return mode
+
     def workspace(self, layer: MoeLayer, n: int, mode: int) -> torch.Tensor:
+        mode = self.effective_mode(layer, n, mode)
         key = (n, mode)
         if key not in layer._ws:
             nbytes = self.lib.ferrite_moe_layer_workspace_bytes(C.byref(layer.shape), n, mode)
@@ -545,11 +557,11 @@ class HipBackend:
 
     def unit_rows(self, layer: MoeLayer, n: int, mode: int = MODE_MFMA_FP8) -> int:
         """Token tile of the expert GEMMs for such a call: 16 (streaming kernels) or 128 (LDS-tiled kernels)."""
-        return int(self.lib.ferrite_moe_layer_unit_rows(C.byref(layer.shape), n, mode))
+        return int(self.lib.ferrite_moe_layer_unit_rows(C.byref(layer.shape), n, self.effective_mode(layer, n, mode)))
 
     def early_experts(self, layer: MoeLayer, n: int, mode: int) -> int:
         """How many routed experts such a call computes ahead of routing on the second stream (0: none)."""
-        return int(self.lib.ferrite_moe_layer_early_experts(C.byref(layer.shape), n, mode))
+        return int(self.lib.ferrite_moe_layer_early_experts(C.byref(layer.shape), n, self.effective_mode(layer, n, mode)))
 
     def moe_layer_dev_mxfp4(self, layer: MoeLayer, x: torch.Tensor, out: torch.Tensor, mode: int = MODE_MFMA_FP8,
                             workspace: Optional[torch.Tensor] = None, stage_events=None, overlap: bool = True):
@@ -569,6 +581,7 @@ class HipBackend:
             raise InvalidArg("x/out must be contiguous f32 or bf16 device tensors")
         if mode != MODE_F32_CHECK and layer.packed is None:
             raise InvalidArg("layer has no packed weights")
+        mode = self.effective_mode(layer, n, mode)   # a declined mode falls back, it is not an error
         ws = workspace if workspace is not None else self.workspace(layer, n, mode)
         self._enter()
         args = (C.byref(layer.shape), C.byref(layer.weights), None if layer.packed is None else layer.packed.data_ptr(),
@@ -604,6 +617,7 @@ class HipBackend:
         self._ck(rc, "moe_layer_mxfp4_static")
 
     def block_workspace(self, layer: MoeLayer, n: int, mode: int) -> torch.Tensor:
+        mode = self.effective_mode(layer, n, mode)
         key = ("block", n, mode)
         if key not in layer._ws:
             nbytes = self.lib.ferrite_moe_block_workspace_bytes(C.byref(layer.shape), n, mode)
@@ -644,6 +658,7 @@ class HipBackend:
             self._dev(t, torch.float32, nm)
         if mode != MODE_F32_CHECK and layer.packed is None:
             raise InvalidArg("layer has no packed weights")
+        mode = self.effective_mode(layer, n, mode)
         ws = workspace if workspace is not None else self.block_workspace(layer, n, mode)
         ptr = lambda t: None if t is None else t.data_ptr()
         blk = MoeBlockArgs(norm_w.data_ptr(), eps, ptr(residual), ptr(post), ptr(comb), nh)
@@ -656,6 +671,7 @@ class HipBackend:
     def workspace_view(self, layer: MoeLayer, n: int, mode: int,
                        workspace: Optional[torch.Tensor] = None) -> Dict[str, torch.Tensor]:
         """Typed views of the intermediates the last layer call left in its workspace."""
+        mode = self.effective_mode(layer, n, mode)
         ws = workspace if workspace is not None else self.workspace(layer, n, mode)
         v = WorkspaceView()
         self._ck(self.lib.ferrite_moe_layer_workspace_view(C.byref(layer.shape), n, mode, ws.data_ptr(), C.byref(v)),

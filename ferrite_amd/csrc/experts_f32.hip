@@ -195,22 +195,35 @@ __global__ __launch_bounds__(256) void combine_kernel(const YT* __restrict__ y, 
     OT* dst = out + (size_t)t * H + h;
     if constexpr (sizeof(OT) == 4) {
         if (hc.residual != nullptr) {
+            // the thread's columns of all nh residual streams first, as hc_post_kernel does: out may then be the
+            // residual buffer itself (the in-place update of the streams)
+            constexpr int MAX_NH = 8;
             const int nh = hc.nh;
-            for (int i = 0; i < nh; ++i) {
+            float rv[MAX_NH][N];
+#pragma unroll
+            for (int k = 0; k < MAX_NH; ++k) {
+                if (k < nh) {
+                    const float* r = hc.residual + ((size_t)t * nh + k) * H + h;
+#pragma unroll
+                    for (int c = 0; c < N; c += 4) {
+                        const float4 q = *reinterpret_cast<const float4*>(r + c);
+                        rv[k][c] = q.x; rv[k][c + 1] = q.y; rv[k][c + 2] = q.z; rv[k][c + 3] = q.w;
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < MAX_NH; ++i) {
+                if (i >= nh) break;
                 const float p = hc.post[(size_t)t * nh + i];
                 float acc[N];
 #pragma unroll
                 for (int c = 0; c < N; ++c) acc[c] = fmul(p, o[c]);
-                for (int k = 0; k < nh; ++k) {
-                    const float cf = hc.comb[((size_t)t * nh + k) * nh + i];
-                    const float* r = hc.residual + ((size_t)t * nh + k) * H + h;
 #pragma unroll
-                    for (int c = 0; c < N; c += 4) {
-                        const float4 rv = *reinterpret_cast<const float4*>(r + c);
-                        acc[c] = fadd(acc[c], fmul(cf, rv.x));
-                        acc[c + 1] = fadd(acc[c + 1], fmul(cf, rv.y));
-                        acc[c + 2] = fadd(acc[c + 2], fmul(cf, rv.z));
-                        acc[c + 3] = fadd(acc[c + 3], fmul(cf, rv.w));
+                for (int k = 0; k < MAX_NH; ++k) {
+                    if (k < nh) {
+                        const float cf = hc.comb[((size_t)t * nh + k) * nh + i];
+#pragma unroll
+                        for (int c = 0; c < N; ++c) acc[c] = fadd(acc[c], fmul(cf, rv[k][c]));
                     }
                 }
                 float* od = reinterpret_cast<float*>(out) + ((size_t)t * nh + i) * H + h;
@@ -251,7 +264,7 @@ int launch_down_f32(const ferrite_moe_shape& s, const ferrite_moe_weights& w, co
 int launch_combine(const void* y, int y_dtype, const float* probs, const int32_t* perm_map, int n, int topk,
                    int hidden, int has_shared, void* out, int out_dtype, hipStream_t st, const HcPostArgs* hcp) {
     const HcPostArgs hc = hcp ? *hcp : HcPostArgs{nullptr, nullptr, nullptr, 0};
-    if (hc.residual && (out_dtype != FERRITE_DT_F32 || hc.nh < 1 || !hc.post || !hc.comb)) return FERRITE_ERR_INVALID_ARG;
+    if (hc.residual && (out_dtype != FERRITE_DT_F32 || hc.nh < 1 || hc.nh > 8 || !hc.post || !hc.comb)) return FERRITE_ERR_INVALID_ARG;
     const bool of32 = out_dtype == FERRITE_DT_F32, yf32 = y_dtype == FERRITE_DT_F32;
     const int per_thread = yf32 ? 4 : 8;   // columns per thread: 16 bytes of a y row
     if (hidden % per_thread) return FERRITE_ERR_INVALID_ARG;

@@ -26,8 +26,9 @@ typedef unsigned int u4v __attribute__((ext_vector_type(4)));  // 128-bit vector
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Which main loop the 128-row units run on (a test hook, ferrite_hip_set_override): 0 = both operands staged
-// through LDS, 1 / 2 = weights streamed into registers by blocks of 4 / 8 waves.
+// Which main loop the 128-row units run on (a test hook, ferrite_hip_set_override): 0 = the faster one for each GEMM
+// (gate/up: weights streamed into registers by blocks of 8 waves; down, whose reduction is a third as long: both
+// operands staged through LDS), 1 = staged for both, 2 / 3 = streamed by blocks of 8 / 4 waves for both.
 static std::atomic<int> g_prefill_variant{0};
 void set_prefill_variant(int v) { g_prefill_variant.store(v, std::memory_order_relaxed); }
 
@@ -1028,10 +1029,7 @@ __device__ __forceinline__ void st_step(const StCtx<W, NT>& c, u4v* lds, int kt,
             if (NB == 1 && tt + 1 < NT) read_tile(tt + 1);
             // Pins the tile: its MFMAs stay in front of this point and the operand reads of the tiles after the next
             // behind it.  Without it the compiler reads all tiles of the step first (64 more registers than there are).
-            if constexpr (NT * 16 > 128)   // 256 accumulators live in the accumulation registers
-                asm volatile("" : "+a"(acc[0][tt]), "+a"(acc[1][tt]), "+a"(acc[2][tt]), "+a"(acc[3][tt]) : : "memory");
-            else
-                asm volatile("" : "+v"(acc[0][tt]), "+v"(acc[1][tt]), "+v"(acc[2][tt]), "+v"(acc[3][tt]) : : "memory");
+            asm volatile("" : "+v"(acc[0][tt]), "+v"(acc[1][tt]), "+v"(acc[2][tt]), "+v"(acc[3][tt]) : : "memory");
         }
     }
     st_load_a(c, min(kt + 3, c.KT - 1), w[R]);
@@ -1223,7 +1221,7 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     if (units.unit_rows_cap >= PF_ROWS) {
         if (x2) return FERRITE_ERR_INVALID_ARG;   // the 128-row kernels take one-term activations
         const int variant = g_prefill_variant.load(std::memory_order_relaxed);
-        if (variant != 0 || units.unit_rows_cap != PF_ROWS) {
+        if (variant != 1 || units.unit_rows_cap != PF_ROWS) {
             auto go = [&](auto kernel, int W, size_t lds) -> int {
                 const int groups = (imax / 32 + W - 1) / W;
                 const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
@@ -1232,17 +1230,13 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
                 return check_launch("gate_up_stream");
             };
             int rc;
-            if (units.unit_rows_cap == 256) {
-                if ((rc = LdsLimit<&gate_up_stream_kernel<4, 16>>::ensure(StCfg<4, 16>::LDS_BYTES))) return rc;
-                return go(gate_up_stream_kernel<4, 16>, 4, StCfg<4, 16>::LDS_BYTES);
-            }
             if (units.unit_rows_cap != PF_ROWS) return FERRITE_ERR_INVALID_ARG;
-            if (variant == 2) {
-                if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
-                return go(gate_up_stream_kernel<8, 8>, 8, StCfg<8, 8>::LDS_BYTES);
+            if (variant == 3) {
+                if ((rc = LdsLimit<&gate_up_stream_kernel<4, 8>>::ensure(StCfg<4, 8>::LDS_BYTES))) return rc;
+                return go(gate_up_stream_kernel<4, 8>, 4, StCfg<4, 8>::LDS_BYTES);
             }
-            if ((rc = LdsLimit<&gate_up_stream_kernel<4, 8>>::ensure(StCfg<4, 8>::LDS_BYTES))) return rc;
-            return go(gate_up_stream_kernel<4, 8>, 4, StCfg<4, 8>::LDS_BYTES);
+            if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
+            return go(gate_up_stream_kernel<8, 8>, 8, StCfg<8, 8>::LDS_BYTES);
         }
         const int groups = (imax / 32 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
@@ -1320,30 +1314,23 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
     if (units.unit_rows_cap >= PF_ROWS) {
         if (x2) return FERRITE_ERR_INVALID_ARG;
         const int variant = g_prefill_variant.load(std::memory_order_relaxed);
-        if (variant != 0 || units.unit_rows_cap != PF_ROWS) {
+        if (variant >= 2 || units.unit_rows_cap != PF_ROWS) {
             auto go = [&](auto kernel, int W, size_t lds, auto* yp) -> int {
                 const int groups = (s.hidden / 64 + W - 1) / W;
                 const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
                 kernel<<<blocks, W * 64, lds, st>>>(a, groups, act.q, act.s, yp);
                 return check_launch("down_stream");
             };
-            int rc;
             const bool bf = y_dtype == FERRITE_DT_BF16;
             uint16_t* yh = static_cast<uint16_t*>(y);
             float* yf = static_cast<float*>(y);
-            if (units.unit_rows_cap == 256) {
-                constexpr size_t lds = StCfg<4, 16>::LDS_BYTES;
-                if ((rc = LdsLimit<&down_stream_kernel<4, 16, uint16_t>>::ensure(lds))) return rc;
-                if ((rc = LdsLimit<&down_stream_kernel<4, 16, float>>::ensure(lds))) return rc;
-                return bf ? go(down_stream_kernel<4, 16, uint16_t>, 4, lds, yh) : go(down_stream_kernel<4, 16, float>, 4, lds, yf);
-            }
             if (units.unit_rows_cap != PF_ROWS) return FERRITE_ERR_INVALID_ARG;
-            if (variant == 2) {
-                constexpr size_t lds = StCfg<8, 8>::LDS_BYTES;
-                return bf ? go(down_stream_kernel<8, 8, uint16_t>, 8, lds, yh) : go(down_stream_kernel<8, 8, float>, 8, lds, yf);
+            if (variant == 3) {
+                constexpr size_t lds = StCfg<4, 8>::LDS_BYTES;
+                return bf ? go(down_stream_kernel<4, 8, uint16_t>, 4, lds, yh) : go(down_stream_kernel<4, 8, float>, 4, lds, yf);
             }
-            constexpr size_t lds = StCfg<4, 8>::LDS_BYTES;
-            return bf ? go(down_stream_kernel<4, 8, uint16_t>, 4, lds, yh) : go(down_stream_kernel<4, 8, float>, 4, lds, yf);
+            constexpr size_t lds = StCfg<8, 8>::LDS_BYTES;
+            return bf ? go(down_stream_kernel<8, 8, uint16_t>, 8, lds, yh) : go(down_stream_kernel<8, 8, float>, 8, lds, yf);
         }
         const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);

@@ -42,11 +42,12 @@ struct Workspace {
 // Process-wide overrides (ferrite_hip_set_override): test hooks that replace what used to be environment reads.
 static std::atomic<int> g_override_unit_rows{0};   // 0 = automatic, else 16 or 128
 static std::atomic<int> g_override_y_f32{0};       // 1 = expert outputs stay f32 on the 128-row path
+static std::atomic<int> g_override_head{0};        // 1 = routing as separate launches whatever the batch size
 static std::atomic<int> g_override_early{0};       // 0 = automatic, k > 0 = k experts ahead of routing, -1 = none
 
 int unit_rows_for(int n, int topk, int n_experts) {
     const int forced = g_override_unit_rows.load(std::memory_order_relaxed);
-    if (forced == 16 || forced == 128 || forced == 256) return forced;
+    if (forced == 16 || forced == 128) return forced;
     return (long)n * topk >= 48L * n_experts ? 128 : 16;
 }
 
@@ -169,8 +170,13 @@ extern "C" const char* ferrite_hip_last_error(void) { return g_last_error; }
 
 extern "C" int ferrite_hip_set_override(int which, int value) {
     if (which == FERRITE_OVERRIDE_UNIT_ROWS) {
-        if (value != 0 && value != 16 && value != 128 && value != 256) return FERRITE_ERR_INVALID_ARG;
+        if (value != 0 && value != 16 && value != 128) return FERRITE_ERR_INVALID_ARG;
         g_override_unit_rows.store(value);
+        return FERRITE_OK;
+    }
+    if (which == FERRITE_OVERRIDE_HEAD) {
+        if (value != 0 && value != 1) return FERRITE_ERR_INVALID_ARG;
+        g_override_head.store(value);
         return FERRITE_OK;
     }
     if (which == FERRITE_OVERRIDE_EARLY_EXPERTS) {
@@ -179,7 +185,7 @@ extern "C" int ferrite_hip_set_override(int which, int value) {
         return FERRITE_OK;
     }
     if (which == FERRITE_OVERRIDE_PREFILL_TILE) {
-        if (value < 0 || value > 2) return FERRITE_ERR_INVALID_ARG;
+        if (value < 0 || value > 3) return FERRITE_ERR_INVALID_ARG;
         set_prefill_variant(value);
         return FERRITE_OK;
     }
@@ -200,6 +206,8 @@ extern "C" int ferrite_hip_warmup(void) {
     void* ws = nullptr;
     return static_workspace(&ws);   // resolves this device's copy of the built-in workspace
 }
+
+extern "C" int ferrite_moe_layer_check(const ferrite_moe_shape* shape, int n, int mode) { return check_shape(shape, n, mode); }
 
 extern "C" int ferrite_moe_layer_unit_rows(const ferrite_moe_shape* shape, int n, int mode) {
     if (check_shape(shape, n, mode)) return 0;
@@ -294,7 +302,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                           const void* x, int x_dtype, int n, void* out, int out_dtype, int mode, void* workspace,
                           size_t workspace_bytes, ferrite_stream_t stream, void* const* ev,
                           const float* norm_w = nullptr, float norm_eps = 0.0f, const HcPostArgs* hc = nullptr,
-                          const OverlapCtx* ov = nullptr) {
+                          const OverlapCtx* ov = nullptr, bool clear_counters = false) {
     int rc = check_shape(shape, n, mode);
     if (rc) return rc;
     // the packed buffer carries the router weight (transposed); the checkpoint-layout one is read only without it
@@ -320,6 +328,13 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
     char* b = static_cast<char*>(workspace);
     hipStream_t st = as_stream(stream);
     const int has_shared = s.shared_inter > 0;
+    if (norm_w && !(packed != nullptr && head_supported(n, s.hidden, s.n_experts) && is_mfma_mode(mode) &&
+                    x_dtype == FERRITE_DT_F32 && head_norm_supported(n, s.hidden, s.n_experts)))
+        return FERRITE_ERR_INVALID_ARG;
+    // every argument has been checked: from here on the call only enqueues
+    if (clear_counters &&
+        (rc = launch_zero_i32(reinterpret_cast<int32_t*>(b + w.counters), n + 1, st)))
+        return rc;
 
     float* logits = reinterpret_cast<float*>(b + w.logits);
     float* probs = reinterpret_cast<float*>(b + w.probs);
@@ -340,7 +355,8 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                      w.max_units};
     units.unit_range = reinterpret_cast<int32_t*>(b + w.unit_range);
     if ((rc = mark(ev, 0, st))) return rc;
-    const bool fused_head = packed != nullptr && head_supported(n, s.hidden, s.n_experts);
+    const bool fused_head = packed != nullptr && head_supported(n, s.hidden, s.n_experts) &&
+                            !(g_override_head.load(std::memory_order_relaxed) == 1 && !norm_w);
     // With a second stream from the caller: quantise x and run gate/up of the first n_early experts and of the shared
     // expert for every token over there, beside the routing head (fork here, join in front of the routed gate/up).
     const bool early = ov != nullptr && w.n_early > 0 && fused_head && is_mfma_mode(mode) && !norm_w;
@@ -470,18 +486,21 @@ static __device__ __align__(256) unsigned char scratch[FERRITE_STATIC_WORKSPACE_
 
 static int static_workspace(void** out) {
     static std::mutex mu;
-    static void* ptrs[kMaxDevices] = {};
+    static std::atomic<void*> ptrs[kMaxDevices] = {};
     int dev = 0;
     if (int rc = current_device(&dev)) return rc;
-    std::lock_guard<std::mutex> lock(mu);
-    if (!ptrs[dev]) {
-        void* p = nullptr;
-        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress");
-        if (!p || (reinterpret_cast<uintptr_t>(p) & 255)) return FERRITE_ERR_RUNTIME;
-        ptrs[dev] = p;
+    void* p = ptrs[dev].load(std::memory_order_acquire);   // the usual case: looked up before, no lock
+    if (!p) {
+        std::lock_guard<std::mutex> lock(mu);
+        p = ptrs[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress");
+            if (!p || (reinterpret_cast<uintptr_t>(p) & 255)) return FERRITE_ERR_RUNTIME;
+            ptrs[dev].store(p, std::memory_order_release);
+        }
     }
-    *out = ptrs[dev];
+    *out = p;
     return FERRITE_OK;
 }
 
@@ -500,11 +519,10 @@ extern "C" int ferrite_moe_layer_mxfp4_static(const ferrite_moe_shape* shape, co
     void* ws = nullptr;
     if ((rc = static_workspace(&ws))) return rc;
     // The array keeps what the last call left in it.  Only the arrival counters have to start at zero; a call that
-    // ran to its end leaves them so, one that was cut short may not have: cleared here, by a kernel (capturable).
-    if ((rc = launch_zero_i32(reinterpret_cast<int32_t*>(static_cast<char*>(ws) + w.counters), n + 1, as_stream(stream))))
-        return rc;
+    // ran to its end leaves them so, one that was cut short may not have: cleared by a kernel (capturable) at the
+    // head of the call's launches, once its arguments have passed every check.
     return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, ws, FERRITE_STATIC_WORKSPACE_BYTES,
-                          stream, nullptr);
+                          stream, nullptr, nullptr, 0.0f, nullptr, nullptr, /*clear_counters=*/true);
 }
 
 // ---- rmsnorm -> layer -> hc_post (exec/lib.rs:487-492) ----
@@ -532,7 +550,10 @@ extern "C" int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const fer
     // The two neighbours fold into the layer's own launches where nothing else needs their results in memory:
     // rmsnorm into the fused routing head (MFMA modes: the expert GEMMs take the quantised activations that the head
     // writes), hc_post into the combine (a per-element function of the layer's output).
-    const bool fused_norm = is_mfma_mode(mode) && packed != nullptr && head_norm_supported(n, s.hidden, s.n_experts);
+    // (the head reads norm_w with 16-byte loads; a misaligned one takes the separate rmsnorm launch, which checks)
+    const bool fused_norm = is_mfma_mode(mode) && packed != nullptr && head_norm_supported(n, s.hidden, s.n_experts) &&
+                            (reinterpret_cast<uintptr_t>(blk->norm_w) & 15) == 0 &&
+                            g_override_head.load(std::memory_order_relaxed) != 1;
     // (hc_post only for decode-sized batches, where it saves a launch: at 4096 tokens the combine with the 4-stream
     // epilogue took 221 us against 57 + 104 us for the two kernels)
     const bool fused_hc = with_hc_post && n <= 256 && blk->nh <= 8 && (reinterpret_cast<uintptr_t>(blk->residual) & 15) == 0;

@@ -65,14 +65,18 @@ int ferrite_hip_warmup(void);
  * the workspace layout: set them before sizing a workspace, not between sizing and use.
  *   FERRITE_OVERRIDE_UNIT_ROWS  0 = automatic (default), 16 or 128 = force that token tile for the expert GEMMs
  *   FERRITE_OVERRIDE_Y_F32      1 = keep the expert outputs `y` in f32 on the 128-row path (default 0: bf16)
- *   FERRITE_OVERRIDE_PREFILL_TILE  main loop of the 128-row units: 0 = default, 1 / 2 = weights streamed into
- *                               registers by blocks of 4 / 8 waves (same bits)
+ *   FERRITE_OVERRIDE_PREFILL_TILE  main loop of the 128-row units: 0 = default (gate/up: weights streamed into
+ *                               registers by blocks of 8 waves; down: both operands staged through LDS), 1 = staged
+ *                               for both GEMMs, 2 / 3 = streamed by blocks of 8 / 4 waves for both (same bits)
  *   FERRITE_OVERRIDE_EARLY_EXPERTS  experts computed ahead of routing by ferrite_moe_layer_mxfp4_ov: 0 = automatic,
- *                               k > 0 = the first k, -1 = none  */
+ *                               k > 0 = the first k, -1 = none
+ *   FERRITE_OVERRIDE_HEAD       1 = router GEMM, routing, permutation and quantisation as separate launches whatever
+ *                               the batch size (default 0: one fused launch for up to 256 tokens)  */
 #define FERRITE_OVERRIDE_UNIT_ROWS 0
 #define FERRITE_OVERRIDE_Y_F32 1
 #define FERRITE_OVERRIDE_PREFILL_TILE 2
 #define FERRITE_OVERRIDE_EARLY_EXPERTS 3
+#define FERRITE_OVERRIDE_HEAD 4
 int ferrite_hip_set_override(int which, int value);
 
 /* ---- KernelBackend ops on the path (f32 device buffers, like the reference's GLM ABI) ---- */
@@ -207,6 +211,12 @@ typedef struct ferrite_moe_workspace_view {
                           * the FERRITE_OVERRIDE_Y_F32 override is off */
 } ferrite_moe_workspace_view;
 
+/* What a layer call with these arguments would answer before it enqueues anything: FERRITE_OK, or
+ * FERRITE_DECLINED (this batch size / shape is outside this mode's contract: the caller falls back to another mode,
+ * as CudaBackend does when a fused kernel declines, cuda.rs:5763-5765,5940,5990 - in particular
+ * FERRITE_MODE_MFMA_FP8_X2 declines prefill-sized batches, whose fallback is FERRITE_MODE_MFMA_FP8), or
+ * FERRITE_ERR_INVALID_ARG.  A declined mode has no workspace size either (ferrite_moe_layer_workspace_bytes is 0). */
+int ferrite_moe_layer_check(const ferrite_moe_shape* shape, int n, int mode);
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
 /* Rows per unit (the token tile of the expert GEMMs) a layer call with these arguments uses: 16 = weights streamed
  * once per unit (decode-sized batches, any activation format),
@@ -255,7 +265,7 @@ int ferrite_moe_layer_mxfp4_ov(const ferrite_moe_shape* shape, const ferrite_moe
 
 /* The same layer for callers that cannot allocate device memory at all and so have no workspace to pass: code
  * under a stream capture that arrives without buffers, tight serving loops, harnesses that forbid hipMalloc.  It has
- * no counterpart in the reference, whose callers always own a DevBuf pool (cuda.rs:558-744).  The workspace is an
+ * no counterpart in the reference.  The workspace is an
  * array of FERRITE_STATIC_WORKSPACE_BYTES built into the library (each GPU the library runs on holds one copy until
  * the process ends); inputs, weights and outputs are still the caller's.  Same results as ferrite_moe_layer_mxfp4,
  * bit for bit.  Calls whose workspace (ferrite_moe_layer_workspace_bytes) exceeds the array return
@@ -292,7 +302,9 @@ int ferrite_hc_post_f32(const float* x, const float* residual, const float* post
  * without hyper-connections, which is also how consecutive layers are chained (out of one = li of the next).  The workspace is the layer's followed by
  * two [n, H] f32 buffers: size it with ferrite_moe_block_workspace_bytes and initialise it once with
  * ferrite_moe_layer_workspace_init (which only touches the layer's part).  Same rules as the layer call: no
- * allocation, no synchronisation, a launch sequence that depends only on (shape, n, mode), capturable. */
+ * allocation, no synchronisation, a launch sequence that depends only on (shape, n, mode), capturable.
+ * Aliasing: out may be the residual buffer itself (the streams updated in place: every thread reads its columns of
+ * all nh streams before it writes any), but must not overlap it in any other way, and must not overlap li. */
 typedef struct {
     const float* norm_w;    /* [H] */
     float eps;
