@@ -29,7 +29,7 @@ ABI_VERSION = 3
 OK, ERR_INVALID_ARG, DECLINED, ERR_WORKSPACE, ERR_RUNTIME = 0, 1, 2, 3, 4
 DT_F32, DT_BF16 = 0, 1
 MODE_F32_CHECK, MODE_MFMA_FP8, MODE_MFMA_FP8_X2 = 0, 1, 2
-OVERRIDE_UNIT_ROWS, OVERRIDE_Y_F32, OVERRIDE_PREFILL_TILE, OVERRIDE_EARLY_EXPERTS, OVERRIDE_HEAD = 0, 1, 2, 3, 4
+OVERRIDE_UNIT_ROWS, OVERRIDE_Y_F32, OVERRIDE_PREFILL_TILE, OVERRIDE_HEAD = 0, 1, 2, 3
 
 
 class FerriteError(RuntimeError):
@@ -90,7 +90,7 @@ EXPORTS = [
     "ferrite_moe_pack_weights", "ferrite_moe_pack_expert", "ferrite_moe_pack_router",
     "ferrite_moe_packed_dequant", "ferrite_moe_layer_workspace_bytes", "ferrite_moe_layer_unit_rows", "ferrite_moe_block_workspace_bytes", "ferrite_moe_block_mxfp4", "ferrite_moe_layer_workspace_init", "ferrite_moe_layer_workspace_view",
     "ferrite_moe_layer_mxfp4", "ferrite_moe_layer_mxfp4_static", "ferrite_moe_layer_mxfp4_timed",
-    "ferrite_moe_layer_check", "ferrite_moe_layer_mxfp4_ov", "ferrite_overlap_create", "ferrite_overlap_destroy", "ferrite_moe_layer_early_experts",
+    "ferrite_moe_layer_check",
     "ferrite_graph_begin", "ferrite_graph_end", "ferrite_graph_launch",
     "ferrite_graph_destroy",
 ]
@@ -137,11 +137,7 @@ def load_library(so_path: Optional[str] = None) -> C.CDLL:
     lib.ferrite_moe_layer_workspace_view.argtypes = [C.POINTER(MoeShape), i32, i32, vp, C.POINTER(WorkspaceView)]
     lib.ferrite_moe_layer_mxfp4.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp, i32, i32, vp, i32,
                                             i32, vp, sz, vp]
-    lib.ferrite_moe_layer_mxfp4_timed.argtypes = lib.ferrite_moe_layer_mxfp4.argtypes + [C.POINTER(vp), vp]
-    lib.ferrite_moe_layer_mxfp4_ov.argtypes = lib.ferrite_moe_layer_mxfp4.argtypes + [vp]
-    lib.ferrite_overlap_create.argtypes = [C.POINTER(vp)]
-    lib.ferrite_overlap_destroy.argtypes = [vp]
-    lib.ferrite_moe_layer_early_experts.argtypes = [C.POINTER(MoeShape), i32, i32]
+    lib.ferrite_moe_layer_mxfp4_timed.argtypes = lib.ferrite_moe_layer_mxfp4.argtypes + [C.POINTER(vp)]
     lib.ferrite_moe_layer_check.argtypes = [C.POINTER(MoeShape), i32, i32]
     lib.ferrite_moe_layer_mxfp4_static.argtypes = [C.POINTER(MoeShape), C.POINTER(MoeWeights), vp, vp, i32, i32, vp, i32,
                                                    i32, vp]
@@ -246,11 +242,8 @@ class HipBackend:
         self._capturing = False
         self._graphs: Dict[str, int] = {}
         self._verify_ok = False
-        self._overrides = {OVERRIDE_UNIT_ROWS: 0, OVERRIDE_Y_F32: 0, OVERRIDE_PREFILL_TILE: 0, OVERRIDE_EARLY_EXPERTS: 0, OVERRIDE_HEAD: 0}
+        self._overrides = {OVERRIDE_UNIT_ROWS: 0, OVERRIDE_Y_F32: 0, OVERRIDE_PREFILL_TILE: 0, OVERRIDE_HEAD: 0}
         self._ck(self.lib.ferrite_hip_warmup(), "warmup")   # LDS limits, before any capture (cuda.rs:627-657)
-        ov = C.c_void_p()
-        self._ck(self.lib.ferrite_overlap_create(C.byref(ov)), "overlap_create")   # the second stream + fork/join events
-        self._overlap = ov
 
     # ---- plumbing ----
     @property
@@ -559,15 +552,10 @@ class HipBackend:
         """Token tile of the expert GEMMs for such a call: 16 (streaming kernels) or 128 (LDS-tiled kernels)."""
         return int(self.lib.ferrite_moe_layer_unit_rows(C.byref(layer.shape), n, self.effective_mode(layer, n, mode)))
 
-    def early_experts(self, layer: MoeLayer, n: int, mode: int) -> int:
-        """How many routed experts such a call computes ahead of routing on the second stream (0: none)."""
-        return int(self.lib.ferrite_moe_layer_early_experts(C.byref(layer.shape), n, self.effective_mode(layer, n, mode)))
-
     def moe_layer_dev_mxfp4(self, layer: MoeLayer, x: torch.Tensor, out: torch.Tensor, mode: int = MODE_MFMA_FP8,
-                            workspace: Optional[torch.Tensor] = None, stage_events=None, overlap: bool = True):
+                            workspace: Optional[torch.Tensor] = None, stage_events=None):
         """The whole layer on the device: router GEMM -> route -> permute -> experts -> combine (+shared).
-        x [n, H] f32 or bf16, out [n, H] f32 or bf16, both pre-allocated device tensors.  overlap: let small batches
-        use the backend's second stream beside the routing head (the same results either way)."""
+        x [n, H] f32 or bf16, out [n, H] f32 or bf16, both pre-allocated device tensors."""
         self.recorder.record("moe_layer_mxfp4")
         self._leave()
         cfg = layer.cfg
@@ -587,13 +575,12 @@ class HipBackend:
         args = (C.byref(layer.shape), C.byref(layer.weights), None if layer.packed is None else layer.packed.data_ptr(),
                 x.data_ptr(), dts[x.dtype], n, out.data_ptr(), dts[out.dtype], mode, ws.data_ptr(), ws.numel(),
                 self._st())
-        ov = self._overlap if overlap else None
         if stage_events is None:
-            self._ck(self.lib.ferrite_moe_layer_mxfp4_ov(*args, ov), "moe_layer_mxfp4")
+            self._ck(self.lib.ferrite_moe_layer_mxfp4(*args), "moe_layer_mxfp4")
         else:
             if len(stage_events) != STAGE_EVENTS:
                 raise InvalidArg(f"stage_events must hold {STAGE_EVENTS} event handles")
-            self._ck(self.lib.ferrite_moe_layer_mxfp4_timed(*args, stage_events, ov), "moe_layer_mxfp4")
+            self._ck(self.lib.ferrite_moe_layer_mxfp4_timed(*args, stage_events), "moe_layer_mxfp4")
 
     def moe_layer_dev_mxfp4_static(self, layer: MoeLayer, x: torch.Tensor, out: torch.Tensor, mode: int = MODE_MFMA_FP8):
         """The same layer on the library's built-in workspace: nothing is allocated, here or in the library."""

@@ -334,9 +334,7 @@ struct MfmaArgs {
     const uint8_t* sh_scales;
     size_t codes_per_expert, scales_per_expert;
     const int32_t *unit_expert, *unit_row0, *unit_rows, *unit_first, *unit_count, *n_units;
-    const int32_t* unit_range;   // [lo, hi): the units this launch covers; NULL = all
     int n, topk, n_experts, hidden, inter, shared_inter, act_ld, unit_cap, max_units;
-    int n_early, dense_row0;     // experts [0, n_early): gate/up results in dense rows dense_row0 + expert * n + token
     float limit;
 };
 
@@ -356,22 +354,16 @@ __device__ __forceinline__ bool unit_ok(const MfmaArgs& a, int e, int row0, int 
 // Used by the 128-row kernels (2-3 units per expert) and by the 16-row kernels (the shared expert's n/16 units, an
 // expert with more than 16 rows).  Returns false for blocks without work or with inconsistent tables.
 __device__ __forceinline__ bool unit_block_work(const MfmaArgs& a, int groups, int& u, int& ig, int& ne) {
-    int lo = 0, hi = min(*a.n_units, a.max_units);
-    if (a.unit_range) {
-        lo = max(a.unit_range[0], 0);
-        hi = min(a.unit_range[1], hi);
-    }
-    const int n_units = hi - lo;
-    if (n_units <= 0) return false;
+    const int n_units = min(*a.n_units, a.max_units);
     const int total = n_units * groups, per_xcd = (total + 7) >> 3;
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int v = xcd * per_xcd + slot;
     if (slot >= per_xcd || v >= total) return false;
-    const int up = lo + v / groups;                  // some unit of the expert whose segment holds v
+    const int up = v / groups;                       // some unit of the expert whose segment holds v
     const int first = a.unit_first[up];
     ne = a.unit_count[up];
-    if (first < lo || ne < 1 || up < first || up >= first + ne || first + ne > hi) return false;
-    const int vl = v - (first - lo) * groups;        // 0 .. ne * groups - 1
+    if (first < 0 || ne < 1 || up < first || up >= first + ne || first + ne > n_units) return false;
+    const int vl = v - first * groups;               // 0 .. ne * groups - 1
     ig = vl / ne;
     u = first + (vl - ig * ne);
     return true;
@@ -488,38 +480,10 @@ __global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gate_up_mfma_k
     else gate_up_unit<WAVES, false, kX2, WIN>(a, u, ig, xin, gather_src, act, lds_raw);
 }
 
-// gate/up of the experts [0, n_early) and of the shared expert for EVERY token, which needs nothing the router
-// produces: it runs beside the routing kernel (whose serial chain leaves HBM idle) and writes dense rows
-// dense_row0 + expert * n + token (the shared expert: its usual rows n * topk + token).  Units are (expert, 16
-// consecutive tokens); blocks map to (expert, item group, token tile) in the XCD-contiguous order of
-// unit_block_work, so the token tiles of one expert read its weights from one L2.  Per token the arithmetic is that
-// of the routed kernel (an MFMA column does not see its neighbours): the same bits.
-template <int WAVES, bool kX2, int WIN>
-__global__ __launch_bounds__(WAVES * 64, WAVES == 4 ? 2 : 1) void gate_up_early_kernel(MfmaArgs a, int groups, ActPlanes xin,
-                                                                                       ActPlanes act) {
-    extern __shared__ __align__(16) unsigned char lds_raw[];
-    const int tiles = (a.n + 15) >> 4;
-    const int experts = a.n_early + (a.shared_inter > 0 ? 1 : 0);
-    const int total = experts * tiles * groups, per_xcd = (total + 7) >> 3;
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int v = xcd * per_xcd + slot;
-    if (slot >= per_xcd || v >= total) return;
-    const int ee = v / (groups * tiles), r = v - ee * (groups * tiles);
-    const int ig = r / tiles, tile = r - ig * tiles;
-    const bool shared = ee >= a.n_early;
-    const int e = shared ? a.n_experts : ee;
-    const int t0 = tile * 16, nrows = min(16, a.n - t0);
-    const int row0 = (shared ? a.n * a.topk : a.dense_row0 + ee * a.n) + t0;
-    auto row_src = [&](int c) -> int { return t0 + c; };
-    if (tiles > 1) gate_up_rows<WAVES, true, kX2, WIN>(a, e, row0, nrows, ig, row_src, xin, act, lds_raw);
-    else gate_up_rows<WAVES, false, kX2, WIN>(a, e, row0, nrows, ig, row_src, xin, act, lds_raw);
-}
-
 // down GEMM: y[row][h] for the unit's rows.  grid: unit_block_work over groups = ceil(items / (WAVES*IPW)); item =
 // 64 rows of H.
 template <int WAVES, int IPW, bool kKeep, bool kX2>
-__device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& act,
-                                          const int32_t* __restrict__ gather_src, float* __restrict__ y,
+__device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, const ActPlanes& act, float* __restrict__ y,
                                           unsigned char* lds_raw) {
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
     if (!unit_ok(a, e, row0, nrows)) return;
@@ -540,17 +504,8 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
     // activation rows have pitch act_ld; only the first `inter` columns are meaningful for this expert
     const BSource<kX2> bsrc{act, (size_t)a.act_ld, scale_pitch(a.act_ld), nrows};
     const int c = lane & 15, g = lane >> 4;
-    // an expert whose gate/up ran ahead of routing keeps its activations in dense rows, one per token
-    const bool dense = e < a.n_early;
-    const int nk = a.n * a.topk, dense0 = a.dense_row0 + e * a.n;
     run_unit<kKeep, kX2, kX2 ? kWindowKt : 0>(
-        bsrc,
-        [&](int col) -> int {
-            if (!dense) return row0 + col;
-            const int i = gather_src[row0 + col];
-            return (i < 0 || i >= nk) ? -1 : dense0 + i / a.topk;
-        },
-        KT, IPW,
+        bsrc, [&](int col) { return row0 + col; }, KT, IPW,
         [&](int r, const u4v*& wp, const u4v*& sp) {
             const int item = item0 + r;
             wp = reinterpret_cast<const u4v*>(cbase) + (size_t)item * KT * 256;
@@ -570,13 +525,12 @@ __device__ __forceinline__ void down_unit(const MfmaArgs& a, int u, int ig, cons
 
 template <int WAVES, int IPW, bool kX2>
 __global__ __launch_bounds__(WAVES * 64, 2) void down_mfma_kernel(MfmaArgs a, int groups, ActPlanes act,
-                                                               const int32_t* __restrict__ gather_src,
                                                                float* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int u, ig, ne;
     if (!unit_block_work(a, groups, u, ig, ne)) return;
-    if (ne > 1) down_unit<WAVES, IPW, true, kX2>(a, u, ig, act, gather_src, y, lds_raw);
-    else down_unit<WAVES, IPW, false, kX2>(a, u, ig, act, gather_src, y, lds_raw);
+    if (ne > 1) down_unit<WAVES, IPW, true, kX2>(a, u, ig, act, y, lds_raw);
+    else down_unit<WAVES, IPW, false, kX2>(a, u, ig, act, y, lds_raw);
 }
 
 
@@ -1203,10 +1157,6 @@ static MfmaArgs make_args(const ferrite_moe_shape& s, const uint8_t* packed, int
     a.limit = s.swiglu_limit;
     a.unit_cap = units.unit_rows_cap;
     a.max_units = units.max_units;
-    a.n_early = units.n_early;
-    a.dense_row0 = units.dense_row0;
-    // the gate/up launch behind the routing kernel leaves out what was computed ahead; down covers every unit
-    a.unit_range = (!down && units.n_early > 0) ? units.unit_range : nullptr;
     return a;
 }
 
@@ -1282,33 +1232,8 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     return check_launch("gate_up_mfma");
 }
 
-// The routing-independent part of gate/up (gate_up_early_kernel): needs the quantised x and nothing else.
-int launch_gate_up_early(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& xin, int n,
-                         const UnitTables& units, const ActPlanes& act, hipStream_t st) {
-    if (units.unit_rows_cap != 16 || units.n_early <= 0) return FERRITE_ERR_INVALID_ARG;
-    MfmaArgs a = make_args(s, packed, n, units, false);
-    a.unit_range = nullptr;
-    const bool x2 = xin.q2 != nullptr;
-    if (x2 != (act.q2 != nullptr)) return FERRITE_ERR_INVALID_ARG;
-    const int KT = s.hidden / 128, imax = a.act_ld;
-    const int groups = (imax / 32 + GU_WAVES - 1) / GU_WAVES;
-    const size_t work = (size_t)(units.n_early + (s.shared_inter > 0 ? 1 : 0)) * ((n + 15) / 16) * groups;
-    const unsigned blocks = (unsigned)((work + 7) / 8 * 8);
-    int rc;
-    if (x2) {
-        const size_t lds = b_lds_bytes<true, kWindowKt>(KT);
-        if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, true, kWindowKt>>::ensure(lds))) return rc;
-        gate_up_early_kernel<GU_WAVES, true, kWindowKt><<<blocks, GU_WAVES * 64, lds, st>>>(a, groups, xin, act);
-    } else {
-        const size_t lds = b_lds_bytes<false, 0>(KT);
-        if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, false, 0>>::ensure(lds))) return rc;
-        gate_up_early_kernel<GU_WAVES, false, 0><<<blocks, GU_WAVES * 64, lds, st>>>(a, groups, xin, act);
-    }
-    return check_launch("gate_up_early");
-}
-
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& act, int n,
-                     const int32_t* gather_src, const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
+                     const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
     MfmaArgs a = make_args(s, packed, n, units, true);
     const bool x2 = act.q2 != nullptr;
     if (units.unit_rows_cap >= PF_ROWS) {
@@ -1344,7 +1269,7 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
         }
         return check_launch("down_prefill");
     }
-    if (units.unit_rows_cap != 16 || (units.n_early > 0 && !gather_src)) return FERRITE_ERR_INVALID_ARG;
+    if (units.unit_rows_cap != 16) return FERRITE_ERR_INVALID_ARG;
     const size_t lds = x2 ? b_lds_bytes<true, kWindowKt>(a.act_ld / 128) : b_lds_bytes<false, 0>(a.act_ld / 128);
     const int items = s.hidden / 64;
     const int groups = (items + DN_WAVES * DN_IPW - 1) / (DN_WAVES * DN_IPW);
@@ -1353,10 +1278,10 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
     int rc;
     if (x2) {
         if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(lds))) return rc;
-        down_mfma_kernel<DN_WAVES, DN_IPW, true><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, gather_src, static_cast<float*>(y));
+        down_mfma_kernel<DN_WAVES, DN_IPW, true><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, static_cast<float*>(y));
     } else {
         if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(lds))) return rc;
-        down_mfma_kernel<DN_WAVES, DN_IPW, false><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, gather_src, static_cast<float*>(y));
+        down_mfma_kernel<DN_WAVES, DN_IPW, false><<<blocks, DN_WAVES * 64, lds, st>>>(a, groups, act, static_cast<float*>(y));
     }
     return check_launch("down_mfma");
 }
@@ -1366,8 +1291,6 @@ int warmup_experts_mfma() {
     if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, false, 0>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES, true, kWindowKt>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES_RESIDENT_X2, true, 0>>::ensure(kLdsCap))) return rc;
-    if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, false, 0>>::ensure(kLdsCap))) return rc;
-    if ((rc = LdsLimit<&gate_up_early_kernel<GU_WAVES, true, kWindowKt>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES))) return rc;

@@ -27,13 +27,6 @@ struct UnitTables {
     int32_t* n_units;      // [1]
     int unit_rows_cap;     // rows per unit (column tile of the GEMM)
     int max_units;
-    // Experts [0, n_early) and the shared expert can be computed ahead of routing, for every token (16-row units
-    // only; 0 = none).  Their gate/up results then live in dense rows dense_row0 + expert * n + token of the
-    // activation buffers, the routing kernels leave in unit_range[0..1] the units [lo, hi) of all other experts, and
-    // the down kernel maps a unit of an early expert to its dense rows.
-    int32_t* unit_range = nullptr;
-    int n_early = 0;
-    int dense_row0 = 0;
 };
 
 inline int max_units_for(int n, int topk, int n_experts, int has_shared, int unit_rows) {
@@ -133,10 +126,8 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
                         const int32_t* gather_src, const UnitTables& units, const ActPlanes& act, hipStream_t st,
                         hipEvent_t k_start = nullptr, hipEvent_t k_stop = nullptr);
 void set_prefill_variant(int v);
-int launch_gate_up_early(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& xin, int n,
-                         const UnitTables& units, const ActPlanes& act, hipStream_t st);
 int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const ActPlanes& act, int n,
-                     const int32_t* gather_src, const UnitTables& units, void* y, int y_dtype, hipStream_t st);
+                     const UnitTables& units, void* y, int y_dtype, hipStream_t st);
 
 // block_ops.hip
 int launch_rmsnorm(const float* x, const float* w, float eps, float* out, int n, int dim, hipStream_t st);

@@ -33,35 +33,20 @@ int check_launch(const char* what) {
 struct Workspace {
     size_t logits, probs, ids_f32, ids, counts, starts, perm_map, gather_src, active, n_active;
     size_t unit_expert, unit_row0, unit_rows, unit_first, unit_count, n_units, perm_scratch, perm_scratch_bytes, counters;
-    size_t xq, xs, xq2, xs2, act, act_s, act2, act_s2, y, unit_range;
+    size_t xq, xs, xq2, xs2, act, act_s, act2, act_s2, y;
     size_t total;
     int max_units, rows, unit_cap;
-    int n_early, act_rows;   // experts whose gate/up may run ahead of routing; rows of the activation buffers
 };
 
 // Process-wide overrides (ferrite_hip_set_override): test hooks that replace what used to be environment reads.
 static std::atomic<int> g_override_unit_rows{0};   // 0 = automatic, else 16 or 128
 static std::atomic<int> g_override_y_f32{0};       // 1 = expert outputs stay f32 on the 128-row path
 static std::atomic<int> g_override_head{0};        // 1 = routing as separate launches whatever the batch size
-static std::atomic<int> g_override_early{0};       // 0 = automatic, k > 0 = k experts ahead of routing, -1 = none
 
 int unit_rows_for(int n, int topk, int n_experts) {
     const int forced = g_override_unit_rows.load(std::memory_order_relaxed);
     if (forced == 16 || forced == 128) return forced;
     return (long)n * topk >= 48L * n_experts ? 128 : 16;
-}
-
-// How many routed experts (the first ones) have their gate/up computed for every token beside the routing kernel
-// when the caller brings a second stream (ferrite_moe_layer_mxfp4_ov): batches of at most 32 tokens, where the
-// routing head is a serial chain that leaves HBM idle for about as long as these experts' weights take to stream.
-// A pure function of (shape, n, mode) like the rest of the workspace layout.
-static int early_experts_for(const ferrite_moe_shape& s, int n, int mode, int unit_cap) {
-    if (!(mode == FERRITE_MODE_MFMA_FP8 || mode == FERRITE_MODE_MFMA_FP8_X2) || unit_cap != 16 || n > 32) return 0;
-    if (!head_supported(n, s.hidden, s.n_experts)) return 0;
-    const int forced = g_override_early.load(std::memory_order_relaxed);
-    if (forced < 0) return 0;
-    const int k = forced > 0 ? forced : 0;   // automatic: none (measured slower at 32 tokens: see the design notes)
-    return k < s.n_experts ? k : s.n_experts - 1;
 }
 
 int y_dtype_for(int unit_rows) {
@@ -120,22 +105,19 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     w.unit_first = bump(off, (size_t)w.max_units * 4);
     w.unit_count = bump(off, (size_t)w.max_units * 4);
     w.n_units = bump(off, 4);
-    w.unit_range = bump(off, 8);
     w.perm_scratch_bytes = perm_scratch_bytes(n, s.n_experts);
     w.perm_scratch = bump(off, w.perm_scratch_bytes);
-    w.n_early = early_experts_for(s, n, mode, w.unit_cap);
-    w.act_rows = w.rows + w.n_early * n;   // dense rows (expert, token) of the experts computed ahead of routing
     if (is_mfma_mode(mode)) {
         const size_t xs_row = ((H / 128 + 3) / 4) * 16, as_row = ((act_ld / 128 + 3) / 4) * 16;
         w.xq = bump(off, (size_t)n * H);
         w.xs = bump(off, (size_t)n * xs_row);
-        w.act = bump(off, (size_t)w.act_rows * act_ld);
-        w.act_s = bump(off, (size_t)w.act_rows * as_row);
+        w.act = bump(off, (size_t)w.rows * act_ld);
+        w.act_s = bump(off, (size_t)w.rows * as_row);
         if (mode == FERRITE_MODE_MFMA_FP8_X2) {
             w.xq2 = bump(off, (size_t)n * H);
             w.xs2 = bump(off, (size_t)n * xs_row);
-            w.act2 = bump(off, (size_t)w.act_rows * act_ld);
-            w.act_s2 = bump(off, (size_t)w.act_rows * as_row);
+            w.act2 = bump(off, (size_t)w.rows * act_ld);
+            w.act_s2 = bump(off, (size_t)w.rows * as_row);
         }
     } else {
         w.act = bump(off, (size_t)w.rows * act_ld * 4);
@@ -177,11 +159,6 @@ extern "C" int ferrite_hip_set_override(int which, int value) {
     if (which == FERRITE_OVERRIDE_HEAD) {
         if (value != 0 && value != 1) return FERRITE_ERR_INVALID_ARG;
         g_override_head.store(value);
-        return FERRITE_OK;
-    }
-    if (which == FERRITE_OVERRIDE_EARLY_EXPERTS) {
-        if (value < -1 || value > 512) return FERRITE_ERR_INVALID_ARG;
-        g_override_early.store(value);
         return FERRITE_OK;
     }
     if (which == FERRITE_OVERRIDE_PREFILL_TILE) {
@@ -251,44 +228,6 @@ extern "C" int ferrite_moe_layer_workspace_view(const ferrite_moe_shape* shape, 
     return FERRITE_OK;
 }
 
-// What a caller brings to let the layer use a second stream: the stream and the two events of the fork and the join.
-struct OverlapCtx {
-    hipStream_t side;
-    hipEvent_t fork, join;
-};
-
-extern "C" int ferrite_overlap_create(void** ctx_out) {
-    if (!ctx_out) return FERRITE_ERR_INVALID_ARG;
-    OverlapCtx* c = new OverlapCtx{};
-    hipError_t e = hipStreamCreateWithFlags(&c->side, hipStreamNonBlocking);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->fork, hipEventDisableTiming);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->join, hipEventDisableTiming);
-    if (e != hipSuccess) {
-        if (c->join) (void)hipEventDestroy(c->join);
-        if (c->fork) (void)hipEventDestroy(c->fork);
-        if (c->side) (void)hipStreamDestroy(c->side);
-        delete c;
-        return hip_fail(e, "ferrite_overlap_create");
-    }
-    *ctx_out = c;
-    return FERRITE_OK;
-}
-
-extern "C" int ferrite_overlap_destroy(void* ctx) {
-    if (!ctx) return FERRITE_OK;
-    OverlapCtx* c = static_cast<OverlapCtx*>(ctx);
-    (void)hipEventDestroy(c->join);
-    (void)hipEventDestroy(c->fork);
-    (void)hipStreamDestroy(c->side);
-    delete c;
-    return FERRITE_OK;
-}
-
-extern "C" int ferrite_moe_layer_early_experts(const ferrite_moe_shape* shape, int n, int mode) {
-    if (check_shape(shape, n, mode)) return 0;
-    return carve(*shape, n, mode).n_early;
-}
-
 static int mark(void* const* ev, int i, hipStream_t st) {
     if (!ev || !ev[i]) return FERRITE_OK;
     hipError_t e = hipEventRecord(static_cast<hipEvent_t>(ev[i]), st);
@@ -302,7 +241,7 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                           const void* x, int x_dtype, int n, void* out, int out_dtype, int mode, void* workspace,
                           size_t workspace_bytes, ferrite_stream_t stream, void* const* ev,
                           const float* norm_w = nullptr, float norm_eps = 0.0f, const HcPostArgs* hc = nullptr,
-                          const OverlapCtx* ov = nullptr, bool clear_counters = false) {
+                          bool clear_counters = false) {
     int rc = check_shape(shape, n, mode);
     if (rc) return rc;
     // the packed buffer carries the router weight (transposed); the checkpoint-layout one is read only without it
@@ -353,26 +292,9 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
                      reinterpret_cast<int32_t*>(b + w.unit_rows), reinterpret_cast<int32_t*>(b + w.unit_first),
                      reinterpret_cast<int32_t*>(b + w.unit_count), reinterpret_cast<int32_t*>(b + w.n_units), w.unit_cap,
                      w.max_units};
-    units.unit_range = reinterpret_cast<int32_t*>(b + w.unit_range);
     if ((rc = mark(ev, 0, st))) return rc;
     const bool fused_head = packed != nullptr && head_supported(n, s.hidden, s.n_experts) &&
                             !(g_override_head.load(std::memory_order_relaxed) == 1 && !norm_w);
-    // With a second stream from the caller: quantise x and run gate/up of the first n_early experts and of the shared
-    // expert for every token over there, beside the routing head (fork here, join in front of the routed gate/up).
-    const bool early = ov != nullptr && w.n_early > 0 && fused_head && is_mfma_mode(mode) && !norm_w;
-    const ActPlanes act_planes = is_mfma_mode(mode)
-                                     ? ActPlanes{at(w.act), at(w.act_s), x2 ? at(w.act2) : nullptr, x2 ? at(w.act_s2) : nullptr}
-                                     : ActPlanes{nullptr, nullptr, nullptr, nullptr};
-    if (early) {
-        units.n_early = w.n_early;
-        units.dense_row0 = w.rows;
-        hipError_t e = hipEventRecord(ov->fork, st);
-        if (e == hipSuccess) e = hipStreamWaitEvent(ov->side, ov->fork, 0);
-        if (e != hipSuccess) return hip_fail(e, "overlap fork");
-        if ((rc = launch_act_quant(x, x_dtype, n, s.hidden, xq.q, xq.s, xq.q2, xq.s2, 1, ov->side))) return rc;
-        if ((rc = launch_gate_up_early(s, packed, xq, n, units, act_planes, ov->side))) return rc;
-        if ((e = hipEventRecord(ov->join, ov->side)) != hipSuccess) return hip_fail(e, "overlap join");
-    }
     if (norm_w && !(fused_head && is_mfma_mode(mode) && x_dtype == FERRITE_DT_F32 &&
                     head_norm_supported(n, s.hidden, s.n_experts)))
         return FERRITE_ERR_INVALID_ARG;
@@ -380,9 +302,8 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         // 1-3 (+ activation quantisation) as one launch
         PackedLayout L = packed_layout(s);
         const int fuse_perm = 1;   // the block that routes the last token builds the tables
-        const ActPlanes head_xq = early ? ActPlanes{nullptr, nullptr, nullptr, nullptr} : xq;   // quantised over there
         if ((rc = launch_moe_head(x, x_dtype, reinterpret_cast<const float*>(packed + L.router_t), wts->router_bias, s,
-                                  n, logits, probs, ids_f32, ids, head_xq, reinterpret_cast<int32_t*>(b + w.counters),
+                                  n, logits, probs, ids_f32, ids, xq, reinterpret_cast<int32_t*>(b + w.counters),
                                   reinterpret_cast<int32_t*>(b + w.counts), reinterpret_cast<int32_t*>(b + w.starts),
                                   perm_map, gather_src, reinterpret_cast<int32_t*>(b + w.active),
                                   reinterpret_cast<int32_t*>(b + w.n_active), &units, fuse_perm, norm_w, norm_eps, st)))
@@ -436,17 +357,13 @@ static int moe_layer_impl(const ferrite_moe_shape* shape, const ferrite_moe_weig
         if ((rc = mark(ev, 5, st))) return rc;
         if ((rc = launch_down_f32(s, *wts, act, n, ids, gather_src, static_cast<float*>(y), st))) return rc;
     } else {
-        const ActPlanes& act = act_planes;
-        if (early) {
-            hipError_t e = hipStreamWaitEvent(st, ov->join, 0);
-            if (e != hipSuccess) return hip_fail(e, "overlap join wait");
-        }
+        const ActPlanes act{at(w.act), at(w.act_s), x2 ? at(w.act2) : nullptr, x2 ? at(w.act_s2) : nullptr};
         if ((rc = launch_gate_up_mfma(s, packed, xq, n, gather_src, units, act, st,
                                       ev ? static_cast<hipEvent_t>(ev[8]) : nullptr,
                                       ev ? static_cast<hipEvent_t>(ev[9]) : nullptr)))
             return rc;
         if ((rc = mark(ev, 5, st))) return rc;
-        if ((rc = launch_down_mfma(s, packed, act, n, gather_src, units, y, y_dtype, st))) return rc;
+        if ((rc = launch_down_mfma(s, packed, act, n, units, y, y_dtype, st))) return rc;
     }
     if ((rc = mark(ev, 6, st))) return rc;
     // 6. weighted combine in slot order + shared expert (exec/lib.rs:1154-1164)
@@ -462,20 +379,12 @@ extern "C" int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const fer
                           nullptr);
 }
 
-extern "C" int ferrite_moe_layer_mxfp4_ov(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
-                                          const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
-                                          int out_dtype, int mode, void* workspace, size_t workspace_bytes,
-                                          ferrite_stream_t stream, void* overlap) {
-    return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, workspace, workspace_bytes, stream,
-                          nullptr, nullptr, 0.0f, nullptr, static_cast<const OverlapCtx*>(overlap));
-}
-
 extern "C" int ferrite_moe_layer_mxfp4_timed(const ferrite_moe_shape* shape, const ferrite_moe_weights* wts,
                                              const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
                                              int out_dtype, int mode, void* workspace, size_t workspace_bytes,
-                                             ferrite_stream_t stream, void* const* stage_events, void* overlap) {
+                                             ferrite_stream_t stream, void* const* stage_events) {
     return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, workspace, workspace_bytes, stream,
-                          stage_events, nullptr, 0.0f, nullptr, static_cast<const OverlapCtx*>(overlap));
+                          stage_events);
 }
 
 // ---- the layer for callers that cannot allocate: its workspace is a file-scope device array ----
@@ -522,7 +431,7 @@ extern "C" int ferrite_moe_layer_mxfp4_static(const ferrite_moe_shape* shape, co
     // ran to its end leaves them so, one that was cut short may not have: cleared by a kernel (capturable) at the
     // head of the call's launches, once its arguments have passed every check.
     return moe_layer_impl(shape, wts, packed, x, x_dtype, n, out, out_dtype, mode, ws, FERRITE_STATIC_WORKSPACE_BYTES,
-                          stream, nullptr, nullptr, 0.0f, nullptr, nullptr, /*clear_counters=*/true);
+                          stream, nullptr, nullptr, 0.0f, nullptr, /*clear_counters=*/true);
 }
 
 // ---- rmsnorm -> layer -> hc_post (exec/lib.rs:487-492) ----

@@ -334,8 +334,6 @@ struct PermArgs {
     int n, topk, n_experts;
     int32_t *counts, *starts, *perm_map, *gather_src, *active, *n_active;
     int32_t *unit_expert, *unit_row0, *unit_rows, *unit_first, *unit_count, *n_units;
-    int32_t* unit_range;   // [2] or NULL: the units [lo, hi) of the experts that are not computed ahead of routing
-    int n_early;           // experts [0, n_early) and the shared expert are (0: none); they own units [0, lo) and [hi, n_units)
     int unit_cap, max_units, has_shared;
 };
 
@@ -375,7 +373,6 @@ __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t*
             ract += c > 0;
             if (a.unit_cap > 0) {
                 const int first = rtile, cnt_e = (c + a.unit_cap - 1) / a.unit_cap;
-                if (a.unit_range && e == a.n_early) a.unit_range[0] = min(first, a.max_units);
                 for (int r = 0; r < c; r += a.unit_cap) {
                     if (rtile < a.max_units) {
                         a.unit_expert[rtile] = e;
@@ -408,13 +405,7 @@ __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t*
                 if (a.unit_first) { a.unit_first[u] = total_tile; a.unit_count[u] = sh_tiles; }
             }
         }
-        if (lane == 0) {
-            *a.n_units = min(total_tile + sh_tiles, a.max_units);
-            if (a.unit_range) {
-                a.unit_range[1] = min(a.n_early > 0 ? total_tile : total_tile + sh_tiles, a.max_units);
-                if (a.n_early >= E) a.unit_range[0] = min(total_tile, a.max_units);
-            }
-        }
+        if (lane == 0) *a.n_units = min(total_tile + sh_tiles, a.max_units);
     }
 }
 
@@ -966,7 +957,6 @@ int launch_moe_head(const void* x, int x_dtype, const float* router_t, const flo
         p.unit_expert = units->unit_expert; p.unit_row0 = units->unit_row0; p.unit_rows = units->unit_rows;
         p.unit_first = units->unit_first; p.unit_count = units->unit_count;
         p.n_units = units->n_units; p.unit_cap = units->unit_rows_cap; p.max_units = units->max_units;
-        p.unit_range = units->unit_range; p.n_early = units->n_early;
     }
     const size_t lds = head_lds_bytes(n, s.hidden, s.n_experts, true);
     if (x_dtype == FERRITE_DT_F32) return launch_head_t<float, true>(a, xq.q ? 1 : 0, lds, st);
@@ -1199,7 +1189,6 @@ int launch_permute(const int32_t* ids, int n, int topk, int n_experts, int32_t* 
         a.unit_expert = units->unit_expert; a.unit_row0 = units->unit_row0; a.unit_rows = units->unit_rows;
         a.unit_first = units->unit_first; a.unit_count = units->unit_count;
         a.n_units = units->n_units; a.unit_cap = units->unit_rows_cap; a.max_units = units->max_units;
-        a.unit_range = units->unit_range; a.n_early = units->n_early;
     }
     const int nchunk = (n + 63) / 64;
     const size_t lds = perm_block_lds_bytes(n, n_experts);

@@ -60,7 +60,7 @@ struct HipBackend::Api {
     FN(ferrite_rmsnorm_f32); FN(ferrite_hc_post_f32);
     FN(ferrite_moe_packed_bytes); FN(ferrite_moe_pack_weights);
     FN(ferrite_moe_layer_workspace_bytes); FN(ferrite_moe_layer_workspace_init); FN(ferrite_moe_layer_mxfp4);
-    FN(ferrite_moe_layer_check); FN(ferrite_moe_layer_mxfp4_ov); FN(ferrite_overlap_create); FN(ferrite_overlap_destroy);
+    FN(ferrite_moe_layer_check);
     FN(ferrite_graph_begin); FN(ferrite_graph_end); FN(ferrite_graph_launch); FN(ferrite_graph_destroy);
 #undef FN
 };
@@ -77,8 +77,7 @@ HipBackend::HipBackend(const std::string& so_path, int device) : api_(new Api) {
     LOAD(ferrite_rmsnorm_f32); LOAD(ferrite_hc_post_f32);
     LOAD(ferrite_moe_packed_bytes); LOAD(ferrite_moe_pack_weights);
     LOAD(ferrite_moe_layer_workspace_bytes); LOAD(ferrite_moe_layer_workspace_init); LOAD(ferrite_moe_layer_mxfp4);
-    LOAD(ferrite_moe_layer_check); LOAD(ferrite_moe_layer_mxfp4_ov); LOAD(ferrite_overlap_create);
-    LOAD(ferrite_overlap_destroy);
+    LOAD(ferrite_moe_layer_check);
     LOAD(ferrite_graph_begin); LOAD(ferrite_graph_end); LOAD(ferrite_graph_launch); LOAD(ferrite_graph_destroy);
 #undef LOAD
     if (api_->ferrite_kernel_abi_version() != FERRITE_ABI_VERSION)
@@ -88,11 +87,9 @@ HipBackend::HipBackend(const std::string& so_path, int device) : api_(new Api) {
     hipck(hipStreamCreate(&s), "hipStreamCreate");   // one stream per backend, default priority
     stream_ = s;
     ck(api_->ferrite_hip_warmup(), "warmup");   // LDS limits, before anything is captured
-    ck(api_->ferrite_overlap_create(&overlap_), "overlap_create");   // the layer's second stream, one per backend
 }
 
 HipBackend::~HipBackend() {
-    if (overlap_) (void)api_->ferrite_overlap_destroy(overlap_);
     if (stream_) (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
     if (so_) dlclose(so_);
 }
@@ -288,9 +285,9 @@ void HipBackend::moe_layer_dev_mxfp4(MoeLayerDev& layer, const DevBuf& x, int x_
         layer.workspace_n = n;
         layer.workspace_mode = mode;
     }
-    ck(api_->ferrite_moe_layer_mxfp4_ov(&layer.shape, &layer.dev, static_cast<const uint8_t*>(layer.packed.ptr), x.ptr,
-                                        x_dtype, n, out.ptr, out_dtype, mode, layer.workspace.ptr, layer.workspace.bytes,
-                                        stream_, overlap_), "moe_layer_mxfp4");
+    ck(api_->ferrite_moe_layer_mxfp4(&layer.shape, &layer.dev, static_cast<const uint8_t*>(layer.packed.ptr), x.ptr,
+                                     x_dtype, n, out.ptr, out_dtype, mode, layer.workspace.ptr, layer.workspace.bytes,
+                                     stream_), "moe_layer_mxfp4");
 }
 
 }  // namespace ferrite

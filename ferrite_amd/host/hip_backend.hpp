@@ -115,7 +115,6 @@ class HipBackend {
     std::unique_ptr<Api> api_;
     void* so_ = nullptr;
     void* stream_ = nullptr;
-    void* overlap_ = nullptr;   // ferrite_overlap_create: the layer's second stream and its fork/join events
     bool capturing_ = false;
     bool verify_ok_ = false;
     std::vector<OpRecord> recorded_;

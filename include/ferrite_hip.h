@@ -68,15 +68,12 @@ int ferrite_hip_warmup(void);
  *   FERRITE_OVERRIDE_PREFILL_TILE  main loop of the 128-row units: 0 = default (gate/up: weights streamed into
  *                               registers by blocks of 8 waves; down: both operands staged through LDS), 1 = staged
  *                               for both GEMMs, 2 / 3 = streamed by blocks of 8 / 4 waves for both (same bits)
- *   FERRITE_OVERRIDE_EARLY_EXPERTS  experts computed ahead of routing by ferrite_moe_layer_mxfp4_ov: 0 = automatic,
- *                               k > 0 = the first k, -1 = none
  *   FERRITE_OVERRIDE_HEAD       1 = router GEMM, routing, permutation and quantisation as separate launches whatever
  *                               the batch size (default 0: one fused launch for up to 256 tokens)  */
 #define FERRITE_OVERRIDE_UNIT_ROWS 0
 #define FERRITE_OVERRIDE_Y_F32 1
 #define FERRITE_OVERRIDE_PREFILL_TILE 2
-#define FERRITE_OVERRIDE_EARLY_EXPERTS 3
-#define FERRITE_OVERRIDE_HEAD 4
+#define FERRITE_OVERRIDE_HEAD 3
 int ferrite_hip_set_override(int which, int value);
 
 /* ---- KernelBackend ops on the path (f32 device buffers, like the reference's GLM ABI) ---- */
@@ -245,24 +242,6 @@ int ferrite_moe_layer_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_we
                             const void* x, int x_dtype, int n, void* out, int out_dtype, int mode,
                             void* workspace, size_t workspace_bytes, ferrite_stream_t stream);
 
-/* The layer with a second stream.  CudaBackend runs its layer on one stream (cuda.rs:996); for batches of at most 32
- * tokens the routing head in front of the expert GEMMs is a serial f32 chain (the reference's summation order,
- * cpu.rs:82-122) that takes about 30 us and leaves HBM idle.  With an overlap context this entry quantises x and
- * runs the gate/up GEMM of the first ferrite_moe_layer_early_experts() routed experts and of the shared expert
- * for EVERY token on the context's stream, beside the routing head (fork after what `stream` holds at the call, join
- * in front of the routed gate/up launch); the routed launch then covers the other experts only, and the down GEMM
- * reads an early expert's activations from dense (expert, token) rows.  The same bits as ferrite_moe_layer_mxfp4.  A
- * graph captured from `stream` records the fork and the join as parallel branches, and the launch sequence
- * still depends on (shape, n, mode) alone.  overlap == NULL, more than 32 tokens, or FERRITE_MODE_F32_CHECK: exactly
- * ferrite_moe_layer_mxfp4.  One context serves one caller at a time (one per backend, like its stream); create and
- * destroy it outside any capture.  No counterpart in the reference. */
-int ferrite_overlap_create(void** overlap_out);
-int ferrite_overlap_destroy(void* overlap);
-int ferrite_moe_layer_early_experts(const ferrite_moe_shape* shape, int n, int mode);
-int ferrite_moe_layer_mxfp4_ov(const ferrite_moe_shape* shape, const ferrite_moe_weights* w, const uint8_t* packed,
-                               const void* x, int x_dtype, int n, void* out, int out_dtype, int mode,
-                               void* workspace, size_t workspace_bytes, ferrite_stream_t stream, void* overlap);
-
 /* The same layer for callers that cannot allocate device memory at all and so have no workspace to pass: code
  * under a stream capture that arrives without buffers, tight serving loops, harnesses that forbid hipMalloc.  It has
  * no counterpart in the reference.  The workspace is an
@@ -325,13 +304,12 @@ int ferrite_moe_block_mxfp4(const ferrite_moe_shape* shape, const ferrite_moe_we
  * after: [1] router GEMM, [2] routing, [3] permutation, [4] activation quantisation (== [3] in f32 mode),
  * [5] gate/up GEMM + SwiGLU, [6] down GEMM, [7] combine; [8] and [9] bracket the gate/up kernel itself on the
  * device (start and end of its execution, without the launch gap that [4]..[5] includes; MFMA mode only).
- * overlap: NULL, or a context as in ferrite_moe_layer_mxfp4_ov ([8] and [9] then bracket the routed gate/up launch,
- * which leaves out the experts computed ahead).  Not capturable. */
+ * Not capturable. */
 #define FERRITE_MOE_STAGE_EVENTS 10
 int ferrite_moe_layer_mxfp4_timed(const ferrite_moe_shape* shape, const ferrite_moe_weights* w,
                                   const uint8_t* packed, const void* x, int x_dtype, int n, void* out,
                                   int out_dtype, int mode, void* workspace, size_t workspace_bytes,
-                                  ferrite_stream_t stream, void* const* stage_events_host, void* overlap);
+                                  ferrite_stream_t stream, void* const* stage_events_host);
 
 /* ---- graph capture: ferrite_graph_begin/end/instantiate/launch (cuda.rs:284-287) ---- */
 int ferrite_graph_begin(ferrite_stream_t stream);

@@ -129,17 +129,35 @@ def test_two_term_long_reductions_stream_their_activations_in_windows(hip, oracl
     check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8, ref32)
 
 
-def test_two_term_mode_is_for_decode_sized_batches(hip):
-    """Prefill-sized batches (n * topk >= 48 * experts) are declined in the two-term mode before anything runs."""
-    from ferrite_amd.backend import Declined, InvalidArg
-    cfg = synth.MoeConfig(200, 256, 8, 3, 256, 128, 4, 2)
-    inp = synth.make_inputs(cfg, seed=1)
+def test_two_term_mode_falls_back_for_prefill_sized_batches(hip, oracle):
+    """Prefill-sized batches (n * topk >= 48 * experts) are declined by the library in the two-term mode before
+    anything runs; the host mirror then does what the reference's caller does with a declined kernel
+    (cuda.rs:5763-5765): it runs the other path.  One layer, one call site, a decode-sized and a prefill-sized batch."""
+    from ferrite_amd.backend import DECLINED, OK
+    import ctypes as C
+    small = synth.MoeConfig(20, 256, 8, 3, 256, 128, 4, 2)
+    inp = synth.make_inputs(small, seed=1)
     layer = hip.load_moe_layer(inp)
-    x = torch.from_numpy(inp.x).to(hip.device)
-    with pytest.raises((Declined, InvalidArg)):
-        hip.moe_layer_dev_mxfp4(layer, x, torch.empty_like(x), MODE_MFMA_FP8_X2)
-    hip.moe_layer_dev_mxfp4(layer, x, torch.empty_like(x), MODE_MFMA_FP8)
-    hip.sync()
+    big = small.with_tokens(200)
+    # the C ABI itself: declined, no workspace size, nothing enqueued
+    assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), 200, MODE_MFMA_FP8_X2) == DECLINED
+    assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), 200, MODE_MFMA_FP8) == OK
+    assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), 20, MODE_MFMA_FP8_X2) == OK
+    assert hip.lib.ferrite_moe_layer_workspace_bytes(C.byref(layer.shape), 200, MODE_MFMA_FP8_X2) == 0
+    assert hip.effective_mode(layer, 20, MODE_MFMA_FP8_X2) == MODE_MFMA_FP8_X2
+    assert hip.effective_mode(layer, 200, MODE_MFMA_FP8_X2) == MODE_MFMA_FP8
+    for cfg, act_mode in ((small, 2), (big, 1)):
+        x_np = synth.make_activations(cfg, seed=3)
+        out, v = run_layer(hip, layer, x_np, MODE_MFMA_FP8_X2)   # the same call for both batch sizes
+        import dataclasses
+        ref = oracle.moe_ffn_mxfp4(dataclasses.replace(inp, cfg=cfg, x=x_np), act_mode=act_mode, n_threads=8)
+        assert np.array_equal(v["ids"], ref["ids"].astype(np.int32))
+        assert max_abs_rel(out, ref["out"]) <= TOL_MFMA
+    # the fallen-back call is the one-term call, bit for bit
+    x_np = synth.make_activations(big, seed=3)
+    a, _ = run_layer(hip, layer, x_np, MODE_MFMA_FP8_X2)
+    b, _ = run_layer(hip, layer, x_np, MODE_MFMA_FP8)
+    assert np.array_equal(a, b)
 
 
 @pytest.fixture
