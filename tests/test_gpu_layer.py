@@ -195,6 +195,36 @@ def test_unit_rows_128_equals_16(hip, oracle, overrides, seed, n, hidden, inter,
     assert max_abs_rel(out_bf16, oracle.moe_ffn_mxfp4(inp, act_mode=1, n_threads=8)["out"]) <= TOL_MFMA_BF16_Y
 
 
+@pytest.mark.parametrize("n,hidden,inter,shared,experts", [(700, 4096, 1536, 1536, 8), (300, 1024, 512, 256, 8),
+                                                           (520, 7168, 2048, 2048, 8)])
+def test_prefill_main_loops_are_bit_identical(hip, overrides, n, hidden, inter, shared, experts):
+    """The 128-row units have two main loops: both operands staged through LDS, or the weights streamed into
+    registers (blocks of 8 or 4 waves) and only the activations staged.  All accumulate over k in the order of the
+    16-row kernels: the same bits at the benchmark's hidden and intermediate sizes (H 4096 / I 1536, H 7168 / I 2048),
+    on full and ragged units, with f32 and with bf16 expert outputs."""
+    from ferrite_amd.backend import OVERRIDE_PREFILL_TILE
+    cfg = synth.MoeConfig(n, hidden, experts, 3, inter, shared, 4 if experts % 4 == 0 else 1, 2 if experts % 4 == 0 else 1)
+    inp = synth.make_inputs(cfg, seed=n)
+    layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
+    try:
+        for y_f32 in (1, 0):
+            outs = {}
+            for rows, variant in ((16, 0), (128, 0), (128, 1), (128, 2), (128, 3)):
+                if rows == 16 and not y_f32:
+                    continue
+                overrides(unit_rows=rows, y_f32=y_f32)
+                hip.set_override(OVERRIDE_PREFILL_TILE, variant)
+                layer._ws.clear()
+                outs[(rows, variant)], v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+                assert int(v["counts"].max()) > 128   # more than one unit per expert, the last one ragged
+            first = next(iter(outs.values()))
+            for k, o in outs.items():
+                assert np.array_equal(o, first), (y_f32, k)
+    finally:
+        hip.set_override(OVERRIDE_PREFILL_TILE, 0)
+        layer._ws.clear()
+
+
 def test_layer_c1_decode(hip, oracle):
     """The decode benchmark shape: 32 tokens, H 4096, 128 experts, top-8 of 8 groups, I 1536, bf16 activations.
     The two-term mode is what the benchmark runs: within 2e-2 of the f32 oracle (CpuBackend's arithmetic)."""
@@ -465,7 +495,7 @@ def test_cpp_host_backend_smoke():
     assert res.returncode == 0 and "ALL OK" in res.stdout
 
 
-def _scale_check(hip, oracle, cfg, n_sample, mode, seed=0):
+def _scale_check(hip, oracle, cfg, n_sample, mode, seed=0, unit_tokens=False):
     """Full-size run: routing and permutation bit-exact for every token, layer output against both oracles on a
     token sample, and a size-independent property: the layer is a per-token function, so permuting the tokens
     permutes the output rows bit for bit."""
@@ -483,6 +513,23 @@ def _scale_check(hip, oracle, cfg, n_sample, mode, seed=0):
           f"mean {counts.mean():.1f}; experts hit {(counts > 0).sum()}")
     assert err <= (TOL_MFMA_BF16_Y if hip.unit_rows(layer, cfg.n, mode) == 128 else TOL_MFMA)
     assert err32 <= (TOL_X2_VS_F32 if mode == MODE_MFMA_FP8_X2 else TOL_X1_VS_F32)
+    if unit_tokens:
+        # Every row of one full unit and of the ragged last unit of one expert at this shape (evenly spaced tokens
+        # touch a unit's first rows at best): the expert whose row count leaves the shortest non-empty last unit
+        # among those with at least one full unit.
+        rows = hip.unit_rows(layer, cfg.n, mode)
+        cand = [e for e in range(cfg.n_experts) if counts[e] > rows and counts[e] % rows]
+        e = min(cand, key=lambda i: counts[i] % rows)
+        start, cnt = int(v["starts"][e]), int(counts[e])
+        last0 = start + (cnt // rows) * rows
+        grouped = np.concatenate([np.arange(start, start + rows), np.arange(last0, start + cnt)])
+        toks = np.unique(v["gather_src"][grouped] // cfg.topk).astype(np.int32)
+        assert len(toks) == len(grouped)   # an expert holds a token once
+        u = oracle.moe_ffn_mxfp4(inp, act_mode=ACT_MODE[mode], n_threads=16, tok_sel=toks)
+        err_u = max_abs_rel(out[toks], u["out"])
+        print(f"{cfg.name}: expert {e} ({cnt} rows): all {rows} rows of its first unit and the {cnt % rows} rows of "
+              f"its last one, {len(toks)} tokens: err {err_u:.3e}")
+        assert err_u <= (TOL_MFMA_BF16_Y if rows == 128 else TOL_MFMA)
     perm = np.random.default_rng(1).permutation(cfg.n)
     out_p, _ = run_layer(hip, layer, inp.x[perm], mode, bf16=cfg.act_bf16)
     assert np.array_equal(out_p, out[perm])
@@ -491,7 +538,7 @@ def _scale_check(hip, oracle, cfg, n_sample, mode, seed=0):
 
 def test_layer_c2_prefill_scale(hip, oracle):
     """4096 tokens, ~256 tokens per expert."""
-    _scale_check(hip, oracle, synth.CONFIGS["c2"], n_sample=12, mode=MODE_MFMA_FP8)
+    _scale_check(hip, oracle, synth.CONFIGS["c2"], n_sample=12, mode=MODE_MFMA_FP8, unit_tokens=True)
 
 
 @pytest.mark.parametrize("mode", [MODE_MFMA_FP8_X2, MODE_MFMA_FP8])
@@ -504,7 +551,7 @@ def test_layer_c3_skewed_scale(hip, oracle):
     """DeepSeek-V3-scale layer with a Zipf(1.1) correction bias: about 10 % of the experts take about half of the
     assignments; stresses the three-phase permutation and experts with thousands of rows."""
     cfg = synth.CONFIGS["c3"]
-    v = _scale_check(hip, oracle, cfg, n_sample=6, mode=MODE_MFMA_FP8)
+    v = _scale_check(hip, oracle, cfg, n_sample=6, mode=MODE_MFMA_FP8, unit_tokens=True)
     counts = np.sort(v["counts"])[::-1]
     top = counts[: cfg.n_experts // 10].sum() / counts.sum()
     assert 0.35 <= top <= 0.65, top
