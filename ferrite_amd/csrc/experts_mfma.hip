@@ -766,11 +766,52 @@ __global__ __launch_bounds__(PF_WAVES * 64, PF_WAVES == 4 ? 2 : 1) void gate_up_
     }
 }
 
-// f32 -> bf16, round to nearest even (NaN stays NaN)
-__device__ __forceinline__ uint32_t bf16_rne(float f) {
-    const uint32_t u = f2u(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+// Two f32 -> two bf16 in one dword, round to nearest even (v_cvt_pk_bf16_f32; NaN stays NaN).
+__device__ __forceinline__ uint32_t bf16_pk(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    const bf2 h = __builtin_convertvector(v, bf2);
+    return *reinterpret_cast<const uint32_t*>(&h);
+}
+
+// Writes the bf16 form of 16 rows x 64 columns of y (one item's columns for one tile of rows): r[t] holds, for the
+// lane's row c = lane % 16, columns 16 t + 4 g .. + 3 with g = lane / 16, as the MFMA leaves them.  Stored from
+// there, a wave's store instruction would put 8 bytes per lane, four 8-byte pieces 32 bytes apart in each of 16
+// rows, and the memory pipeline takes as long per such piece as per full line: at 4096 tokens the stores of
+// the 128-row down kernel cost 83 us of its 291 us.  So the pieces change lanes first: two lane-row swaps
+// (v_permlane32_swap, v_permlane16_swap) per dword pair hand lane (c, g) the 16 bytes at columns 8 g and the 16
+// bytes at columns 32 + 8 g of its row, then neighbouring rows trade their second halves (DPP quad_perm), and each
+// of the two store instructions writes eight whole 128-byte rows: 243 us.  `y_row0` points at column 0 of the item
+// in the row of c = 0; rows c >= rows_here are not written.  Every lane of the wave must call this.
+__device__ __forceinline__ void store_y_tile_bf16(uint16_t* __restrict__ y_row0, size_t pitch, int rows_here, v4f r0,
+                                                  v4f r1, v4f r2, v4f r3, int lane) {
+    typedef unsigned u2v __attribute__((ext_vector_type(2)));
+    const int c = lane & 15, g = lane >> 4;
+    uint32_t lo[4] = {bf16_pk(r0[0], r0[1]), bf16_pk(r1[0], r1[1]), bf16_pk(r2[0], r2[1]), bf16_pk(r3[0], r3[1])};
+    uint32_t hi[4] = {bf16_pk(r0[2], r0[3]), bf16_pk(r1[2], r1[3]), bf16_pk(r2[2], r2[3]), bf16_pk(r3[2], r3[3])};
+    // lane rows g = 0..3 of registers (t, t+1): [t0 t1 t2 t3] [u0 u1 u2 u3] -> [t0 t2 u0 u2] [t1 t3 u1 u3]
+#pragma unroll
+    for (int p = 0; p < 4; p += 2) {
+        u2v a = __builtin_amdgcn_permlane32_swap(lo[p], lo[p + 1], false, false);
+        a = __builtin_amdgcn_permlane16_swap(a[0], a[1], false, false);
+        u2v b = __builtin_amdgcn_permlane32_swap(hi[p], hi[p + 1], false, false);
+        b = __builtin_amdgcn_permlane16_swap(b[0], b[1], false, false);
+        lo[p] = a[0]; lo[p + 1] = a[1]; hi[p] = b[0]; hi[p + 1] = b[1];
+    }
+    // now (lo[0], hi[0], lo[1], hi[1]) = columns 8 g .. 8 g + 7 and (lo[2], hi[2], lo[3], hi[3]) = columns 32 + 8 g ..
+    const uint32_t q0 = __builtin_amdgcn_update_dpp(0u, lo[2], 0xB1, 0xf, 0xf, false);   // lane ^ 1's second half
+    const uint32_t q1 = __builtin_amdgcn_update_dpp(0u, hi[2], 0xB1, 0xf, 0xf, false);
+    const uint32_t q2 = __builtin_amdgcn_update_dpp(0u, lo[3], 0xB1, 0xf, 0xf, false);
+    const uint32_t q3 = __builtin_amdgcn_update_dpp(0u, hi[3], 0xB1, 0xf, 0xf, false);
+    const bool even = (c & 1) == 0;
+    // first store: the even row of each pair, its first half from the even lane, its second half from the odd lane
+    const u4v sa = {even ? lo[0] : q0, even ? hi[0] : q1, even ? lo[1] : q2, even ? hi[1] : q3};
+    const u4v sb = {even ? q0 : lo[0], even ? q1 : hi[0], even ? q2 : lo[1], even ? q3 : hi[1]};
+    const int ra = c & ~1, rb = c | 1;
+    const int first = g * 8, second = 32 + g * 8;
+    if (ra < rows_here) *reinterpret_cast<u4v*>(y_row0 + (size_t)ra * pitch + (even ? first : second)) = sa;
+    if (rb < rows_here) *reinterpret_cast<u4v*>(y_row0 + (size_t)rb * pitch + (even ? second : first)) = sb;
 }
 
 template <typename YT>
@@ -801,18 +842,20 @@ __global__ __launch_bounds__(PF_WAVES * 64, PF_WAVES == 4 ? 2 : 1) void down_pre
         if (item >= items) break;
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-            const int col = (c.wt * 4 + tt) * 16 + cc;
-            if (col < nrows) {
-                YT* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
+            const int tile0 = (c.wt * 4 + tt) * 16;
+            if constexpr (sizeof(YT) == 4) {
+                const int col = tile0 + cc;
+                if (col < nrows) {
+                    YT* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const v4f r = acc[ii][t][tt];
-                    if constexpr (sizeof(YT) == 4)
+                    for (int t = 0; t < 4; ++t) {
+                        const v4f r = acc[ii][t][tt];
                         *reinterpret_cast<float4*>(dst + t * 16) = make_float4(r[0], r[1], r[2], r[3]);
-                    else
-                        *reinterpret_cast<uint2*>(dst + t * 16) =
-                            make_uint2(bf16_rne(r[0]) | (bf16_rne(r[1]) << 16), bf16_rne(r[2]) | (bf16_rne(r[3]) << 16));
+                    }
                 }
+            } else {
+                store_y_tile_bf16(y + (size_t)(row0 + tile0) * H + (size_t)item * 64, (size_t)H, nrows - tile0,
+                                  acc[ii][0][tt], acc[ii][1][tt], acc[ii][2][tt], acc[ii][3][tt], c.lane);
             }
         }
     }
@@ -1117,18 +1160,19 @@ __global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void down_stream_kern
 #pragma unroll
     for (int tt = 0; tt < NT; ++tt) {
         if (tt >= c.ntile) continue;
-        const int col = tt * 16 + cc;
-        if (col < nrows) {
-            YT* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
+        if constexpr (sizeof(YT) == 4) {
+            const int col = tt * 16 + cc;
+            if (col < nrows) {
+                YT* dst = y + (size_t)(row0 + col) * H + (size_t)item * 64 + g * 4;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const v4f r = acc[t][tt];
-                if constexpr (sizeof(YT) == 4)
+                for (int t = 0; t < 4; ++t) {
+                    const v4f r = acc[t][tt];
                     *reinterpret_cast<float4*>(dst + t * 16) = make_float4(r[0], r[1], r[2], r[3]);
-                else
-                    *reinterpret_cast<uint2*>(dst + t * 16) =
-                        make_uint2(bf16_rne(r[0]) | (bf16_rne(r[1]) << 16), bf16_rne(r[2]) | (bf16_rne(r[3]) << 16));
+                }
             }
+        } else {
+            store_y_tile_bf16(y + (size_t)(row0 + tt * 16) * H + (size_t)item * 64, (size_t)H, nrows - tt * 16, acc[0][tt],
+                              acc[1][tt], acc[2][tt], acc[3][tt], c.lane);
         }
     }
 }

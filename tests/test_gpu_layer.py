@@ -225,6 +225,34 @@ def test_prefill_main_loops_are_bit_identical(hip, overrides, n, hidden, inter, 
         layer._ws.clear()
 
 
+@pytest.mark.parametrize("variant", [0, 2])
+def test_prefill_bf16_expert_rows_are_the_rounded_f32_rows(hip, overrides, variant):
+    """The 128-row down kernels hand the expert outputs to the combine step as bf16: packed hardware conversion, then
+    an exchange between lanes so that a store instruction writes whole rows.  Every value must be the round-to-
+    nearest-even of the f32 value the same kernel writes under the test override (torch's cast states the rounding),
+    in full and in ragged units, for the LDS-staged and the weight-streaming kernel."""
+    from ferrite_amd.backend import OVERRIDE_PREFILL_TILE
+    cfg = synth.MoeConfig(700, 1024, 8, 3, 512, 256, 4, 2)
+    inp = synth.make_inputs(cfg, seed=11)
+    layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
+    try:
+        hip.set_override(OVERRIDE_PREFILL_TILE, variant)
+        ys = {}
+        for y_f32 in (1, 0):
+            overrides(unit_rows=128, y_f32=y_f32)
+            layer._ws.clear()
+            _, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+            assert int(v["counts"].max()) > 128 and int(v["counts"].min()) % 16 != 0
+            ys[y_f32] = v["y"].copy()   # f32 as written, or the bf16 values widened (exact)
+        assert np.isfinite(ys[1]).all() and float(np.abs(ys[1]).max()) > 0
+        rounded = torch.from_numpy(ys[1]).to(torch.bfloat16).float().numpy()
+        assert not np.array_equal(rounded, ys[1])                       # the f32 run really kept more bits
+        assert np.array_equal(rounded.view(np.uint32), ys[0].view(np.uint32))
+    finally:
+        hip.set_override(OVERRIDE_PREFILL_TILE, 0)
+        layer._ws.clear()
+
+
 def test_layer_c1_decode(hip, oracle):
     """The decode benchmark shape: 32 tokens, H 4096, 128 experts, top-8 of 8 groups, I 1536, bf16 activations.
     The two-term mode is what the benchmark runs: within 2e-2 of the f32 oracle (CpuBackend's arithmetic)."""
