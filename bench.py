@@ -425,7 +425,7 @@ def main():
         px_np = synth.make_activations(pcfg, seed=0)
         px = torch.from_numpy(px_np).to(hip.device).to(torch.bfloat16)
         pmode = hip.effective_mode(layer, pn, asked)
-        pl = layer_leg(hip, torch, ev, layer, px, pn, pcfg, pmode, max(10, min(50, args.steps)), 5, stack=False)
+        pl = layer_leg(hip, torch, ev, layer, px, pn, pcfg, pmode, max(10, min(50, args.steps)), 20, stack=False)
         pcounts = pl["counts"]
         pab = algorithmic_bytes(pcfg, pn, int((pcounts > 0).sum()))
         pflops = 2.0 * pn * (pcfg.topk * pcfg.inter + pcfg.shared_inter) * 3 * pcfg.hidden
