@@ -526,11 +526,17 @@ class HipBackend:
     def effective_mode(self, layer: MoeLayer, n: int, mode: int) -> int:
         """The mode a layer call for n tokens runs in: the one asked for, or, where the library declines it, the mode
         the caller falls back to (cuda.rs:5763-5765: a declined fused kernel is not an error, the other path runs).
-        Two-term activations are declined for prefill-sized batches: those run with one term."""
-        rc = self.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, mode)
-        if rc == DECLINED and mode == MODE_MFMA_FP8_X2 and \
-                self.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, MODE_MFMA_FP8) == OK:
-            return MODE_MFMA_FP8
+        The order is two-term MFMA -> one-term MFMA -> the f32 mode; the MFMA modes decline shapes whose hidden or
+        intermediate size is not a multiple of 128, which the f32 mode serves from the checkpoint-layout weights."""
+        chain = [MODE_MFMA_FP8_X2, MODE_MFMA_FP8, MODE_F32_CHECK]
+        if mode not in chain:
+            return mode
+        for m in chain[chain.index(mode):]:
+            rc = self.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, m)
+            if rc == OK:
+                return m
+            if rc != DECLINED:
+                break
         return mode
 
     def workspace(self, layer: MoeLayer, n: int, mode: int) -> torch.Tensor:
@@ -567,9 +573,9 @@ class HipBackend:
         dts = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
         if x.dtype not in dts or out.dtype not in dts or not x.is_contiguous() or not out.is_contiguous():
             raise InvalidArg("x/out must be contiguous f32 or bf16 device tensors")
+        mode = self.effective_mode(layer, n, mode)   # a declined mode falls back, it is not an error
         if mode != MODE_F32_CHECK and layer.packed is None:
             raise InvalidArg("layer has no packed weights")
-        mode = self.effective_mode(layer, n, mode)   # a declined mode falls back, it is not an error
         ws = workspace if workspace is not None else self.workspace(layer, n, mode)
         self._enter()
         args = (C.byref(layer.shape), C.byref(layer.weights), None if layer.packed is None else layer.packed.data_ptr(),
@@ -673,7 +679,7 @@ class HipBackend:
             return ws[off:off + count * size].view(dtype)
 
         E, k = cfg.n_experts, cfg.topk
-        y_bf16 = (mode != MODE_F32_CHECK and self.unit_rows(layer, n, mode) >= 128
+        y_bf16 = (mode != MODE_F32_CHECK and self.unit_rows(layer, n, mode) >= 64
                   and not self._overrides[OVERRIDE_Y_F32])
         y_dtype = torch.bfloat16 if y_bf16 else torch.float32
         return dict(logits=view(v.logits, n * E, torch.float32).view(n, E),

@@ -545,6 +545,7 @@ __global__ __launch_bounds__(WAVES * 64, 2) void down_mfma_kernel(MfmaArgs a, in
 // barrier, operand reads) hides behind the other's MFMAs.
 // Accumulation order over k is the same as in the 16-row kernels, so both give the same bits.
 constexpr int PF_ROWS = 128;
+constexpr int PF_ROWS_X2 = 64;                         // two-term activations: half the rows, both planes of each
 constexpr int PF_ITEMS = 4;                            // 8 (one block of 8 waves per CU) is correct too and measured slower
 constexpr int PF_WAVES = PF_ITEMS;                     // one wave per item for the fills; 2 items x 64 rows each for the MFMAs
 constexpr int PF_A_SLOTS = PF_ITEMS * 256;             // u4v of weights per stage
@@ -907,8 +908,12 @@ struct StCtx {
     int KT, lane, wave, ntile, bslot;
 };
 
-// row_q(col) / row_s(col): byte offsets of unit column col's code row / scale row from bq / bs.
-template <int W, int NT, typename RowQ, typename RowS>
+// A stage holds NT operand tiles of 16 rows each.  With one-term activations tile v is rows 16 v .. 16 v + 15 of the
+// unit; with two-term activations (P = 2 planes) the unit has NT / 2 tiles of rows and tile v is plane v % 2 of row
+// tile v / 2: both planes of a row tile accumulate into the same registers, and the tiles that hold rows of the unit
+// are the first ones of the stage in either case.
+// row_q(v, r) / row_s(v, r): byte offsets of row r of tile v's code row / scale row from bq / bs.
+template <int P, int W, int NT, typename RowQ, typename RowS>
 __device__ __forceinline__ void st_context(StCtx<W, NT>& c, const uint8_t* cbase, const uint8_t* sbase, int item, int KT,
                                            int nrows, const uint8_t* bq, size_t bq_bytes, const uint8_t* bs,
                                            size_t bs_bytes, RowQ row_q, RowS row_s) {
@@ -917,7 +922,7 @@ __device__ __forceinline__ void st_context(StCtx<W, NT>& c, const uint8_t* cbase
     c.KT = KT;
     c.lane = threadIdx.x & 63;
     c.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    c.ntile = min(NT, (nrows + 15) >> 4);
+    c.ntile = min(NT / P, (nrows + 15) >> 4);
     c.ra = make_rsrc(cbase + (size_t)item * KT * 4096, (size_t)KT * 4096);
     c.ras = make_rsrc(sbase + (size_t)item * KT4 * 1024, (size_t)KT4 * 1024);
     c.rb = make_rsrc(bq, bq_bytes);
@@ -929,14 +934,10 @@ __device__ __forceinline__ void st_context(StCtx<W, NT>& c, const uint8_t* cbase
 #pragma unroll
     for (int i = 0; i < Cfg::CF; ++i) {
         const int j = c.wave * Cfg::CF + i;
-        const int col = (j >> 1) * 16 + (c.lane >> 2);
-        c.coff[i] = row_q(col < nrows ? col : 0) + (uint32_t)((j & 1) * 64 + ((c.lane & 3) ^ ((c.lane >> 3) & 3)) * 16);
+        c.coff[i] = row_q(j >> 1, c.lane >> 2) + (uint32_t)((j & 1) * 64 + ((c.lane & 3) ^ ((c.lane >> 3) & 3)) * 16);
     }
 #pragma unroll
-    for (int i = 0; i < Cfg::SF; ++i) {
-        const int col = min(c.wave * Cfg::SF + i, NT - 1) * 16 + cc;
-        c.soff[i] = row_s(col < nrows ? col : 0) + (uint32_t)(g * 4);
-    }
+    for (int i = 0; i < Cfg::SF; ++i) c.soff[i] = row_s(min(c.wave * Cfg::SF + i, NT - 1), cc) + (uint32_t)(g * 4);
     c.bslot = 4 * cc + (g ^ ((cc >> 1) & 3));
 }
 
@@ -984,9 +985,9 @@ __device__ __forceinline__ void st_load_a(const StCtx<W, NT>& c, int kt, StWeigh
 // used): a load behind a branch makes the compiler wait for all loads at the next use of any.
 // kFull: all NT tiles of rows are live; otherwise tiles beyond ntile get no MFMAs (a unit's last block of rows is
 // usually far from full).
-template <int R, bool kFull, int W, int NT>
+template <int R, bool kFull, int P, int W, int NT>
 __device__ __forceinline__ void st_step(const StCtx<W, NT>& c, u4v* lds, int kt, StWeights (&w)[3], StFill<W, NT>& f,
-                                        v4f (&acc)[4][NT]) {
+                                        v4f (&acc)[4][NT / P]) {
     using Cfg = StCfg<W, NT>;
     __syncthreads();   // stage R is complete; nobody reads the stage that is written next any more
     st_store(c, lds + ((R + 1) % 3) * Cfg::STAGE_SLOTS, f);
@@ -1012,7 +1013,8 @@ __device__ __forceinline__ void st_step(const StCtx<W, NT>& c, u4v* lds, int kt,
     read_tile(0);
 #pragma unroll
     for (int tt = 0; tt < NT; ++tt) {
-        if (kFull || tt < c.ntile) {   // block-uniform
+        const int rt = tt / P;
+        if (kFull || rt < c.ntile) {   // block-uniform; the live tiles are the first ones
             if (NB == 2 && tt + 1 < NT) read_tile(tt + 1);
             const u4v b0 = b[tt % NB][0], b1 = b[tt % NB][1];
             bs[tt % NB] >>= sh;
@@ -1020,37 +1022,37 @@ __device__ __forceinline__ void st_step(const StCtx<W, NT>& c, u4v* lds, int kt,
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                 const v8i a8 = {(int)w[R].a[t][0], (int)w[R].a[t][1], (int)w[R].a[t][2], (int)w[R].a[t][3], 0, 0, 0, 0};
-                acc[t][tt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, bv, acc[t][tt], 4 /*A e2m1*/, 0 /*B e4m3*/,
+                acc[t][rt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, bv, acc[t][rt], 4 /*A e2m1*/, 0 /*B e4m3*/,
                                                                               0, (int)w[R].sc[t], 0, (int)bs[tt % NB]);
             }
             if (NB == 1 && tt + 1 < NT) read_tile(tt + 1);
             // Pins the tile: its MFMAs stay in front of this point and the operand reads of the tiles after the next
             // behind it.  Without it the compiler reads all tiles of the step first (64 more registers than there are).
-            asm volatile("" : "+v"(acc[0][tt]), "+v"(acc[1][tt]), "+v"(acc[2][tt]), "+v"(acc[3][tt]) : : "memory");
+            asm volatile("" : "+v"(acc[0][rt]), "+v"(acc[1][rt]), "+v"(acc[2][rt]), "+v"(acc[3][rt]) : : "memory");
         }
     }
     st_load_a(c, min(kt + 3, c.KT - 1), w[R]);
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool kFull, int W, int NT>
+template <bool kFull, int P, int W, int NT>
 __device__ __forceinline__ void st_steps(const StCtx<W, NT>& c, u4v* lds, StWeights (&w)[3], StFill<W, NT>& f,
-                                         v4f (&acc)[4][NT]) {
+                                         v4f (&acc)[4][NT / P]) {
     const int KT = c.KT;
     int kt = 0;
 #pragma unroll 1
     for (; kt + 3 <= KT; kt += 3) {
-        st_step<0, kFull>(c, lds, kt, w, f, acc);
-        st_step<1, kFull>(c, lds, kt + 1, w, f, acc);
-        st_step<2, kFull>(c, lds, kt + 2, w, f, acc);
+        st_step<0, kFull, P>(c, lds, kt, w, f, acc);
+        st_step<1, kFull, P>(c, lds, kt + 1, w, f, acc);
+        st_step<2, kFull, P>(c, lds, kt + 2, w, f, acc);
     }
     const int rem = KT - kt;   // block-uniform
-    if (rem > 0) st_step<0, kFull>(c, lds, kt, w, f, acc);
-    if (rem > 1) st_step<1, kFull>(c, lds, kt + 1, w, f, acc);
+    if (rem > 0) st_step<0, kFull, P>(c, lds, kt, w, f, acc);
+    if (rem > 1) st_step<1, kFull, P>(c, lds, kt + 1, w, f, acc);
 }
 
-template <int W, int NT>
-__device__ __forceinline__ void st_mainloop(const StCtx<W, NT>& c, u4v* lds, v4f (&acc)[4][NT]) {
+template <int P, int W, int NT>
+__device__ __forceinline__ void st_mainloop(const StCtx<W, NT>& c, u4v* lds, v4f (&acc)[4][NT / P]) {
     const int KT = c.KT;
     StWeights w[3];
 #pragma unroll
@@ -1060,17 +1062,35 @@ __device__ __forceinline__ void st_mainloop(const StCtx<W, NT>& c, u4v* lds, v4f
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int tt = 0; tt < NT; ++tt) acc[t][tt] = (v4f){0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < NT / P; ++tt) acc[t][tt] = (v4f){0.f, 0.f, 0.f, 0.f};
     st_store(c, lds, f);
     st_load(c, min(1, KT - 1), f);
-    st_steps<false>(c, lds, w, f, acc);
+    st_steps<false, P>(c, lds, w, f, acc);
 }
 
-template <int W, int NT>
+// The span of two planes that one buffer resource covers: plane p starts d[p] bytes after lo.
+struct PlaneSpan {
+    const uint8_t* lo;
+    uint32_t d0, d1;
+    size_t bytes;
+    __device__ __forceinline__ uint32_t at(int plane) const { return plane ? d1 : d0; }
+};
+__device__ __forceinline__ PlaneSpan plane_span(const uint8_t* p0, const uint8_t* p1, size_t plane_bytes) {
+    if (!p1) return PlaneSpan{p0, 0u, 0u, plane_bytes};
+    const uint8_t* lo = p0 < p1 ? p0 : p1;
+    const uint32_t d0 = (uint32_t)(p0 - lo), d1 = (uint32_t)(p1 - lo);
+    return PlaneSpan{lo, d0, d1, (size_t)(d0 > d1 ? d0 : d1) + plane_bytes};
+}
+
+// P = 1: one-term activations, units of up to NT * 16 rows.  P = 2: two-term activations (both planes of x in, both
+// planes of the SwiGLU output out), units of up to NT * 8 rows: per k step and tile of rows a second MFMA against
+// the second plane with the same weight registers, so the stage, the fills and the MFMAs per block are those of
+// P = 1 and a launch has twice the blocks.
+template <int W, int NT, int P>
 __global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void gate_up_stream_kernel(
-    MfmaArgs a, int groups, const uint8_t* __restrict__ xq, const uint8_t* __restrict__ xs,
-    const int32_t* __restrict__ gather_src, uint8_t* __restrict__ act_q, uint8_t* __restrict__ act_s) {
+    MfmaArgs a, int groups, ActPlanes xin, const int32_t* __restrict__ gather_src, ActPlanes act) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
+    constexpr int RT = NT / P;
     int u, ig, ne;
     if (!unit_block_work(a, groups, u, ig, ne)) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
@@ -1082,28 +1102,31 @@ __global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void gate_up_stream_k
     const int H = a.hidden, nk = a.n * a.topk, topk = a.topk, n = a.n;
     const int spitch = scale_pitch(H);
     auto token = [&](int col) -> int {
-        const int gr = row0 + col;
+        const int gr = row0 + (col < nrows ? col : 0);
         if (shared) return gr - nk;
         const int i = gather_src[gr];
         const int tk = (i < 0 || i >= nk) ? 0 : i / topk;
         return tk < n ? tk : 0;
     };
+    const PlaneSpan xq = plane_span(xin.q, P == 2 ? xin.q2 : nullptr, (size_t)n * H);
+    const PlaneSpan xs = plane_span(xin.s, P == 2 ? xin.s2 : nullptr, (size_t)n * spitch);
     StCtx<W, NT> c;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int item = item0 + wave;
-    st_context(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
-               shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), H / 128, nrows, xq,
-               (size_t)n * H, xs, (size_t)n * spitch, [&](int col) { return (uint32_t)token(col) * (uint32_t)H; },
-               [&](int col) { return (uint32_t)token(col) * (uint32_t)spitch; });
-    v4f acc[4][NT];
-    st_mainloop(c, reinterpret_cast<u4v*>(lds_raw), acc);
+    st_context<P>(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
+                  shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), H / 128, nrows,
+                  xq.lo, xq.bytes, xs.lo, xs.bytes,
+                  [&](int v, int r) { return xq.at(v % P) + (uint32_t)token((v / P) * 16 + r) * (uint32_t)H; },
+                  [&](int v, int r) { return xs.at(v % P) + (uint32_t)token((v / P) * 16 + r) * (uint32_t)spitch; });
+    v4f acc[4][RT];
+    st_mainloop<P>(c, reinterpret_cast<u4v*>(lds_raw), acc);
     if (item >= items) return;
 
     // tiles 0,1 = gate rows [0,16),[16,32) of the item; tiles 2,3 = the same up rows
     const int cc = c.lane & 15, g = c.lane >> 4;
     const int apitch = scale_pitch(a.act_ld);
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt) {
+    for (int tt = 0; tt < RT; ++tt) {
         if (tt >= c.ntile) continue;
         const int col = tt * 16 + cc;
         float r0[4], r1[4];
@@ -1116,25 +1139,47 @@ __global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void gate_up_stream_k
         }
         amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
         amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        const uint32_t sb = block_scale_e8m0(amax);
+        const float inv = u2f((254u - sb) << 23);
+        const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
+        const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
+        const size_t qoff = (size_t)(row0 + col) * a.act_ld + (size_t)item * 32 + g * 4;
+        const size_t soff = (size_t)(row0 + col) * apitch + scale_pos(item);
         if (col < nrows) {
-            const uint32_t sb = block_scale_e8m0(amax);
-            const float inv = u2f((254u - sb) << 23);
-            const uint32_t p0 = e4m3_encode4_hw(r0[0] * inv, r0[1] * inv, r0[2] * inv, r0[3] * inv);
-            const uint32_t p1 = e4m3_encode4_hw(r1[0] * inv, r1[1] * inv, r1[2] * inv, r1[3] * inv);
-            uint8_t* dst = act_q + (size_t)(row0 + col) * a.act_ld + (size_t)item * 32 + g * 4;
-            *reinterpret_cast<uint32_t*>(dst) = p0;
-            *reinterpret_cast<uint32_t*>(dst + 16) = p1;
-            if (g == 0) act_s[(size_t)(row0 + col) * apitch + scale_pos(item)] = (uint8_t)sb;
+            *reinterpret_cast<uint32_t*>(act.q + qoff) = p0;
+            *reinterpret_cast<uint32_t*>(act.q + qoff + 16) = p1;
+            if (g == 0) act.s[soff] = (uint8_t)sb;
+        }
+        if constexpr (P == 2) {
+            // second term: the same quantiser on what the first leaves over (as in the 16-row kernel)
+            const float sc = u2f(sb << 23);
+            float amax2 = 0.0f;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                r0[v] = fadd(r0[v], -fmul(e4m3_decode((p0 >> (8 * v)) & 0xffu), sc));
+                r1[v] = fadd(r1[v], -fmul(e4m3_decode((p1 >> (8 * v)) & 0xffu), sc));
+                amax2 = fmaxf(amax2, fmaxf(fabsf(r0[v]), fabsf(r1[v])));
+            }
+            amax2 = fmaxf(amax2, __shfl_xor(amax2, 16, 64));
+            amax2 = fmaxf(amax2, __shfl_xor(amax2, 32, 64));
+            const uint32_t sb2 = block_scale_e8m0(amax2);
+            const float inv2 = u2f((254u - sb2) << 23);
+            const uint32_t t0 = e4m3_encode4_hw(r0[0] * inv2, r0[1] * inv2, r0[2] * inv2, r0[3] * inv2);
+            const uint32_t t1 = e4m3_encode4_hw(r1[0] * inv2, r1[1] * inv2, r1[2] * inv2, r1[3] * inv2);
+            if (col < nrows) {
+                *reinterpret_cast<uint32_t*>(act.q2 + qoff) = t0;
+                *reinterpret_cast<uint32_t*>(act.q2 + qoff + 16) = t1;
+                if (g == 0) act.s2[soff] = (uint8_t)sb2;
+            }
         }
     }
 }
 
-template <int W, int NT, typename YT>
-__global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void down_stream_kernel(MfmaArgs a, int groups,
-                                                                                   const uint8_t* __restrict__ act_q,
-                                                                                   const uint8_t* __restrict__ act_s,
+template <int W, int NT, int P, typename YT>
+__global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void down_stream_kernel(MfmaArgs a, int groups, ActPlanes act,
                                                                                    YT* __restrict__ y) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
+    constexpr int RT = NT / P;
     int u, ig, ne;
     if (!unit_block_work(a, groups, u, ig, ne)) return;
     const int e = a.unit_expert[u], row0 = a.unit_row0[u], nrows = a.unit_rows[u];
@@ -1144,21 +1189,27 @@ __global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void down_stream_kern
     const int H = a.hidden, items = H / 64, item0 = ig * W;
     if (item0 >= items) return;
     const int apitch = scale_pitch(a.act_ld), act_ld = a.act_ld;
+    // both planes from the unit's first row on: the resources end with the unit's last row
+    const PlaneSpan aq = plane_span(act.q + (size_t)row0 * act_ld, P == 2 ? act.q2 + (size_t)row0 * act_ld : nullptr,
+                                    (size_t)nrows * act_ld);
+    const PlaneSpan as = plane_span(act.s + (size_t)row0 * apitch, P == 2 ? act.s2 + (size_t)row0 * apitch : nullptr,
+                                    (size_t)nrows * apitch);
     StCtx<W, NT> c;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int item = item0 + wave;
-    st_context(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
-               shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), inter / 128, nrows,
-               act_q + (size_t)row0 * act_ld, (size_t)nrows * act_ld, act_s + (size_t)row0 * apitch, (size_t)nrows * apitch,
-               [&](int col) { return (uint32_t)col * (uint32_t)act_ld; },
-               [&](int col) { return (uint32_t)col * (uint32_t)apitch; });
-    v4f acc[4][NT];
-    st_mainloop(c, reinterpret_cast<u4v*>(lds_raw), acc);
+    auto rowc = [&](int v, int r) { const int col = (v / P) * 16 + r; return (uint32_t)(col < nrows ? col : 0); };
+    st_context<P>(c, shared ? a.sh_codes : a.codes + (size_t)e * a.codes_per_expert,
+                  shared ? a.sh_scales : a.scales + (size_t)e * a.scales_per_expert, min(item, items - 1), inter / 128, nrows,
+                  aq.lo, aq.bytes, as.lo, as.bytes,
+                  [&](int v, int r) { return aq.at(v % P) + rowc(v, r) * (uint32_t)act_ld; },
+                  [&](int v, int r) { return as.at(v % P) + rowc(v, r) * (uint32_t)apitch; });
+    v4f acc[4][RT];
+    st_mainloop<P>(c, reinterpret_cast<u4v*>(lds_raw), acc);
     if (item >= items) return;
 
     const int cc = c.lane & 15, g = c.lane >> 4;
 #pragma unroll
-    for (int tt = 0; tt < NT; ++tt) {
+    for (int tt = 0; tt < RT; ++tt) {
         if (tt >= c.ntile) continue;
         if constexpr (sizeof(YT) == 4) {
             const int col = tt * 16 + cc;
@@ -1178,6 +1229,12 @@ __global__ __launch_bounds__(W * 64, W * NT <= 32 ? 2 : 1) void down_stream_kern
 }
 
 // ---- launchers ----------------------------------------------------------------------------------------
+// true when two planes of `bytes` each can be addressed from the lower one with 32-bit offsets
+static bool planes_within_4g(const uint8_t* p0, const uint8_t* p1, size_t bytes) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p0), b = reinterpret_cast<uintptr_t>(p1);
+    return (a > b ? a - b : b - a) + bytes < 0xffffffffull;
+}
+
 constexpr int GU_WAVES = 4;
 constexpr int GU_WAVES_RESIDENT_X2 = 8;
 constexpr int DN_WAVES = 4;
@@ -1212,30 +1269,36 @@ int launch_gate_up_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const
     const int imax = a.act_ld;
     const bool x2 = xin.q2 != nullptr;
     if (x2 != (act.q2 != nullptr)) return FERRITE_ERR_INVALID_ARG;
-    if (units.unit_rows_cap >= PF_ROWS) {
-        if (x2) return FERRITE_ERR_INVALID_ARG;   // the 128-row kernels take one-term activations
+    if (units.unit_rows_cap >= PF_ROWS_X2) {
+        // the tiled kernels: 128-row units of one-term activations, 64-row units of two-term activations
+        if (units.unit_rows_cap != (x2 ? PF_ROWS_X2 : PF_ROWS)) return FERRITE_ERR_INVALID_ARG;
         const int variant = g_prefill_variant.load(std::memory_order_relaxed);
-        if (variant != 1 || units.unit_rows_cap != PF_ROWS) {
-            auto go = [&](auto kernel, int W, size_t lds) -> int {
-                const int groups = (imax / 32 + W - 1) / W;
-                const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-                hipExtLaunchKernelGGL(kernel, dim3(blocks), dim3(W * 64), (uint32_t)lds, st, k_start, k_stop, 0, a, groups,
-                                      xin.q, xin.s, gather_src, act.q, act.s);
-                return check_launch("gate_up_stream");
-            };
-            int rc;
-            if (units.unit_rows_cap != PF_ROWS) return FERRITE_ERR_INVALID_ARG;
-            if (variant == 3) {
-                if ((rc = LdsLimit<&gate_up_stream_kernel<4, 8>>::ensure(StCfg<4, 8>::LDS_BYTES))) return rc;
-                return go(gate_up_stream_kernel<4, 8>, 4, StCfg<4, 8>::LDS_BYTES);
-            }
-            if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
-            return go(gate_up_stream_kernel<8, 8>, 8, StCfg<8, 8>::LDS_BYTES);
+        auto go = [&](auto kernel, int W, size_t lds) -> int {
+            const int groups = (imax / 32 + W - 1) / W;
+            const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+            hipExtLaunchKernelGGL(kernel, dim3(blocks), dim3(W * 64), (uint32_t)lds, st, k_start, k_stop, 0, a, groups,
+                                  xin, gather_src, act);
+            return check_launch("gate_up_stream");
+        };
+        int rc;
+        if (x2) {
+            // both planes through one buffer resource each: 32-bit offsets
+            if (!planes_within_4g(xin.q, xin.q2, (size_t)n * s.hidden) || !planes_within_4g(xin.s, xin.s2, (size_t)n * scale_pitch(s.hidden)))
+                return FERRITE_ERR_INVALID_ARG;
+            if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8, 2>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
+            return go(gate_up_stream_kernel<8, 8, 2>, 8, StCfg<8, 8>::LDS_BYTES);
+        }
+        if (variant == 3) {
+            if ((rc = LdsLimit<&gate_up_stream_kernel<4, 8, 1>>::ensure(StCfg<4, 8>::LDS_BYTES))) return rc;
+            return go(gate_up_stream_kernel<4, 8, 1>, 4, StCfg<4, 8>::LDS_BYTES);
+        }
+        if (variant != 1) {
+            if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8, 1>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
+            return go(gate_up_stream_kernel<8, 8, 1>, 8, StCfg<8, 8>::LDS_BYTES);
         }
         const int groups = (imax / 32 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-        int rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES);
-        if (rc) return rc;
+        if ((rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES))) return rc;
         hipExtLaunchKernelGGL(gate_up_prefill_kernel, dim3(blocks), dim3(PF_WAVES * 64), (uint32_t)PF_LDS_BYTES, st, k_start,
                               k_stop, 0, a, groups, xin.q, xin.s, gather_src, act.q, act.s);
         return check_launch("gate_up_prefill");
@@ -1280,36 +1343,42 @@ int launch_down_mfma(const ferrite_moe_shape& s, const uint8_t* packed, const Ac
                      const UnitTables& units, void* y, int y_dtype, hipStream_t st) {
     MfmaArgs a = make_args(s, packed, n, units, true);
     const bool x2 = act.q2 != nullptr;
-    if (units.unit_rows_cap >= PF_ROWS) {
-        if (x2) return FERRITE_ERR_INVALID_ARG;
+    if (units.unit_rows_cap >= PF_ROWS_X2) {
+        if (units.unit_rows_cap != (x2 ? PF_ROWS_X2 : PF_ROWS)) return FERRITE_ERR_INVALID_ARG;
         const int variant = g_prefill_variant.load(std::memory_order_relaxed);
-        if (variant >= 2 || units.unit_rows_cap != PF_ROWS) {
-            auto go = [&](auto kernel, int W, size_t lds, auto* yp) -> int {
-                const int groups = (s.hidden / 64 + W - 1) / W;
-                const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
-                kernel<<<blocks, W * 64, lds, st>>>(a, groups, act.q, act.s, yp);
-                return check_launch("down_stream");
-            };
-            const bool bf = y_dtype == FERRITE_DT_BF16;
-            uint16_t* yh = static_cast<uint16_t*>(y);
-            float* yf = static_cast<float*>(y);
-            if (units.unit_rows_cap != PF_ROWS) return FERRITE_ERR_INVALID_ARG;
-            if (variant == 3) {
-                constexpr size_t lds = StCfg<4, 8>::LDS_BYTES;
-                return bf ? go(down_stream_kernel<4, 8, uint16_t>, 4, lds, yh) : go(down_stream_kernel<4, 8, float>, 4, lds, yf);
-            }
+        const bool bf = y_dtype == FERRITE_DT_BF16;
+        uint16_t* yh = static_cast<uint16_t*>(y);
+        float* yf = static_cast<float*>(y);
+        auto go = [&](auto kernel, int W, size_t lds, auto* yp) -> int {
+            const int groups = (s.hidden / 64 + W - 1) / W;
+            const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
+            kernel<<<blocks, W * 64, lds, st>>>(a, groups, act, yp);
+            return check_launch("down_stream");
+        };
+        if (x2) {
+            const size_t rows = (size_t)n * s.topk + (s.shared_inter > 0 ? n : 0);
+            if (!planes_within_4g(act.q, act.q2, rows * a.act_ld) || !planes_within_4g(act.s, act.s2, rows * scale_pitch(a.act_ld)))
+                return FERRITE_ERR_INVALID_ARG;
             constexpr size_t lds = StCfg<8, 8>::LDS_BYTES;
-            return bf ? go(down_stream_kernel<8, 8, uint16_t>, 8, lds, yh) : go(down_stream_kernel<8, 8, float>, 8, lds, yf);
+            return bf ? go(down_stream_kernel<8, 8, 2, uint16_t>, 8, lds, yh) : go(down_stream_kernel<8, 8, 2, float>, 8, lds, yf);
+        }
+        if (variant == 3) {
+            constexpr size_t lds = StCfg<4, 8>::LDS_BYTES;
+            return bf ? go(down_stream_kernel<4, 8, 1, uint16_t>, 4, lds, yh) : go(down_stream_kernel<4, 8, 1, float>, 4, lds, yf);
+        }
+        if (variant == 2) {
+            constexpr size_t lds = StCfg<8, 8>::LDS_BYTES;
+            return bf ? go(down_stream_kernel<8, 8, 1, uint16_t>, 8, lds, yh) : go(down_stream_kernel<8, 8, 1, float>, 8, lds, yf);
         }
         const int groups = (s.hidden / 64 + PF_ITEMS - 1) / PF_ITEMS;
         const unsigned blocks = (unsigned)(((size_t)units.max_units * groups + 7) / 8 * 8);
         int rc;
-        if (y_dtype == FERRITE_DT_BF16) {
+        if (bf) {
             if ((rc = LdsLimit<&down_prefill_kernel<uint16_t>>::ensure(PF_LDS_BYTES))) return rc;
-            down_prefill_kernel<uint16_t><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act.q, act.s, static_cast<uint16_t*>(y));
+            down_prefill_kernel<uint16_t><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act.q, act.s, yh);
         } else {
             if ((rc = LdsLimit<&down_prefill_kernel<float>>::ensure(PF_LDS_BYTES))) return rc;
-            down_prefill_kernel<float><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act.q, act.s, static_cast<float*>(y));
+            down_prefill_kernel<float><<<blocks, PF_WAVES * 64, PF_LDS_BYTES, st>>>(a, groups, act.q, act.s, yf);
         }
         return check_launch("down_prefill");
     }
@@ -1337,6 +1406,8 @@ int warmup_experts_mfma() {
     if ((rc = LdsLimit<&gate_up_mfma_kernel<GU_WAVES_RESIDENT_X2, true, 0>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, false>>::ensure(kLdsCap))) return rc;
     if ((rc = LdsLimit<&down_mfma_kernel<DN_WAVES, DN_IPW, true>>::ensure(kLdsCap))) return rc;
+    if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8, 1>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
+    if ((rc = LdsLimit<&gate_up_stream_kernel<8, 8, 2>>::ensure(StCfg<8, 8>::LDS_BYTES))) return rc;
     if ((rc = LdsLimit<&gate_up_prefill_kernel>::ensure(PF_LDS_BYTES))) return rc;
     if ((rc = LdsLimit<&down_prefill_kernel<uint16_t>>::ensure(PF_LDS_BYTES))) return rc;
     return LdsLimit<&down_prefill_kernel<float>>::ensure(PF_LDS_BYTES);

@@ -43,14 +43,19 @@ static std::atomic<int> g_override_unit_rows{0};   // 0 = automatic, else 16 or 
 static std::atomic<int> g_override_y_f32{0};       // 1 = expert outputs stay f32 on the 128-row path
 static std::atomic<int> g_override_head{0};        // 1 = routing as separate launches whatever the batch size
 
-int unit_rows_for(int n, int topk, int n_experts) {
+// Rows per unit: 16 (the weight-streaming kernels) for decode-sized batches; for prefill-sized ones the tiled
+// kernels, whose units hold 128 rows of one-term or 64 rows of two-term activations.  The override forces one
+// family or the other (16, or 128 = the tiled kernels).
+int unit_rows_for(int n, int topk, int n_experts, bool two_term) {
+    const int tiled = two_term ? 64 : 128;
     const int forced = g_override_unit_rows.load(std::memory_order_relaxed);
-    if (forced == 16 || forced == 128) return forced;
-    return (long)n * topk >= 48L * n_experts ? 128 : 16;
+    if (forced == 16) return 16;
+    if (forced == 128) return tiled;
+    return (long)n * topk >= 48L * n_experts ? tiled : 16;
 }
 
 int y_dtype_for(int unit_rows) {
-    if (unit_rows < 128) return FERRITE_DT_F32;
+    if (unit_rows < 64) return FERRITE_DT_F32;
     return g_override_y_f32.load(std::memory_order_relaxed) ? FERRITE_DT_F32 : FERRITE_DT_BF16;
 }
 
@@ -85,7 +90,7 @@ static Workspace carve(const ferrite_moe_shape& s, int n, int mode) {
     const int has_shared = s.shared_inter > 0;
     const size_t act_ld = s.inter > s.shared_inter ? s.inter : s.shared_inter;
     w.rows = (int)(nk + (has_shared ? n : 0));
-    w.unit_cap = mode == FERRITE_MODE_MFMA_FP8 ? unit_rows_for(n, s.topk, s.n_experts) : 16;
+    w.unit_cap = is_mfma_mode(mode) ? unit_rows_for(n, s.topk, s.n_experts, mode == FERRITE_MODE_MFMA_FP8_X2) : 16;
     w.max_units = max_units_for(n, s.topk, s.n_experts, has_shared, w.unit_cap);
     size_t off = 0;
     w.counters = bump(off, ((size_t)n + 1) * 4);   // first: ferrite_moe_layer_workspace_init clears it
@@ -135,8 +140,6 @@ static int check_shape(const ferrite_moe_shape* s, int n, int mode) {
     if (mode != FERRITE_MODE_F32_CHECK && !is_mfma_mode(mode)) return FERRITE_ERR_INVALID_ARG;
     if (s->hidden % 32 || s->inter % 32 || s->shared_inter % 32) return FERRITE_ERR_INVALID_ARG;
     if (is_mfma_mode(mode) && (s->hidden % 128 || s->inter % 128 || s->shared_inter % 128)) return FERRITE_DECLINED;
-    // two-term activations exist for the weight-streaming kernels only (decode-sized batches)
-    if (mode == FERRITE_MODE_MFMA_FP8_X2 && (long)n * s->topk >= 48L * s->n_experts) return FERRITE_DECLINED;
     if (n > 65535) return FERRITE_DECLINED;   // token index on grid.y of several kernels: split the batch
     // the routing kernels' own limits, for the fused head and the separate launches alike
     return check_routing_params(s->n_experts, s->topk, s->n_group, s->topk_group);

@@ -271,11 +271,19 @@ void HipBackend::moe_layer_dev_mxfp4(MoeLayerDev& layer, const DevBuf& x, int x_
     const size_t esz_x = x_dtype == FERRITE_DT_F32 ? 4 : 2, esz_o = out_dtype == FERRITE_DT_F32 ? 4 : 2;
     if (x.bytes < (size_t)n * layer.shape.hidden * esz_x) throw FerriteError(FerriteError::ShapeMismatch, "x too small");
     if (out.bytes < (size_t)n * layer.shape.hidden * esz_o) throw FerriteError(FerriteError::InvalidArg, "out too small");
-    // A mode that declines this batch is not an error: the caller falls back (cuda.rs:5763-5765,5926-5937).  Two-term
-    // activations are for decode-sized batches; a prefill-sized one runs the same layer with one term.
-    if (mode == FERRITE_MODE_MFMA_FP8_X2 && api_->ferrite_moe_layer_check(&layer.shape, n, mode) == FERRITE_DECLINED &&
-        api_->ferrite_moe_layer_check(&layer.shape, n, FERRITE_MODE_MFMA_FP8) == FERRITE_OK)
-        mode = FERRITE_MODE_MFMA_FP8;
+    // A mode that declines this call is not an error: the caller falls back (cuda.rs:5763-5765,5926-5937), two-term
+    // MFMA -> one-term MFMA -> the f32 mode (the MFMA modes decline hidden / intermediate sizes that are not
+    // multiples of 128; the f32 mode serves those from the checkpoint-layout weights).
+    {
+        const int chain[3] = {FERRITE_MODE_MFMA_FP8_X2, FERRITE_MODE_MFMA_FP8, FERRITE_MODE_F32_CHECK};
+        int at = 0;
+        while (at < 3 && chain[at] != mode) ++at;
+        for (int i = at; i < 3; ++i) {
+            const int rc = api_->ferrite_moe_layer_check(&layer.shape, n, chain[i]);
+            if (rc == FERRITE_OK) { mode = chain[i]; break; }
+            if (rc != FERRITE_DECLINED) break;
+        }
+    }
     if (layer.workspace_n != n || layer.workspace_mode != mode) {
         if (capturing_) throw FerriteError(FerriteError::InvalidArg, "workspace must be sized before capture");
         const size_t wb = api_->ferrite_moe_layer_workspace_bytes(&layer.shape, n, mode);

@@ -39,7 +39,7 @@ def check_mfma(hip, oracle, layer, inp, mode, ref32=None, bf16=False, n_threads=
         check_routing(v, ref32, oracle, inp.cfg)
     refq = oracle.moe_ffn_mxfp4(inp, act_mode=ACT_MODE[mode], n_threads=n_threads)
     err_q, err_32 = max_abs_rel(out, refq["out"]), max_abs_rel(out, ref32["out"])
-    tol_q = TOL_MFMA_BF16_Y if hip.unit_rows(layer, inp.cfg.n, mode) == 128 else TOL_MFMA
+    tol_q = TOL_MFMA_BF16_Y if hip.unit_rows(layer, inp.cfg.n, mode) >= 64 else TOL_MFMA
     assert err_q <= tol_q, (mode, err_q)
     assert err_32 <= (TOL_X2_VS_F32 if mode == MODE_MFMA_FP8_X2 else TOL_X1_VS_F32), (mode, err_32)
     return out, v, err_q, err_32
@@ -129,35 +129,46 @@ def test_two_term_long_reductions_stream_their_activations_in_windows(hip, oracl
     check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8, ref32)
 
 
-def test_two_term_mode_falls_back_for_prefill_sized_batches(hip, oracle):
-    """Prefill-sized batches (n * topk >= 48 * experts) are declined by the library in the two-term mode before
-    anything runs; the host mirror then does what the reference's caller does with a declined kernel
-    (cuda.rs:5763-5765): it runs the other path.  One layer, one call site, a decode-sized and a prefill-sized batch."""
+def test_declined_mode_falls_back(hip, oracle):
+    """A shape the MFMA modes decline (hidden size not a multiple of 128) is declined before anything runs; the host
+    mirror then does what the reference's caller does with a declined kernel (cuda.rs:5763-5765): it runs the other
+    path, here the f32 mode on the checkpoint-layout weights.  One layer, one call site, a decode-sized and a
+    prefill-sized batch; and the two-term mode itself serves both sizes of a shape it accepts."""
     from ferrite_amd.backend import DECLINED, OK
     import ctypes as C
+    import dataclasses
+    odd = synth.MoeConfig(20, 160, 8, 3, 96, 64, 4, 2)
+    inp = synth.make_inputs(odd, seed=1)
+    layer = hip.load_moe_layer(inp, pack=False)
+    for n in (20, 200):
+        # the C ABI itself: declined, no workspace size, nothing enqueued
+        assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, MODE_MFMA_FP8_X2) == DECLINED
+        assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, MODE_MFMA_FP8) == DECLINED
+        assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, MODE_F32_CHECK) == OK
+        assert hip.lib.ferrite_moe_layer_workspace_bytes(C.byref(layer.shape), n, MODE_MFMA_FP8_X2) == 0
+        assert hip.effective_mode(layer, n, MODE_MFMA_FP8_X2) == MODE_F32_CHECK
+        cfg = odd.with_tokens(n)
+        x_np = synth.make_activations(cfg, seed=3)
+        out, v = run_layer(hip, layer, x_np, MODE_MFMA_FP8_X2)   # the same call for both batch sizes
+        ref = oracle.moe_ffn_mxfp4(dataclasses.replace(inp, cfg=cfg, x=x_np), n_threads=8)
+        check_routing(v, ref, oracle, cfg)
+        assert max_abs_rel(out, ref["out"]) <= TOL_F32
+        direct, _ = run_layer(hip, layer, x_np, MODE_F32_CHECK)
+        assert np.array_equal(out, direct)                     # the fallen-back call is the f32 call, bit for bit
+    # a shape the MFMA modes accept: two-term activations at a decode-sized and at a prefill-sized batch
     small = synth.MoeConfig(20, 256, 8, 3, 256, 128, 4, 2)
     inp = synth.make_inputs(small, seed=1)
     layer = hip.load_moe_layer(inp)
-    big = small.with_tokens(200)
-    # the C ABI itself: declined, no workspace size, nothing enqueued
-    assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), 200, MODE_MFMA_FP8_X2) == DECLINED
-    assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), 200, MODE_MFMA_FP8) == OK
-    assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), 20, MODE_MFMA_FP8_X2) == OK
-    assert hip.lib.ferrite_moe_layer_workspace_bytes(C.byref(layer.shape), 200, MODE_MFMA_FP8_X2) == 0
-    assert hip.effective_mode(layer, 20, MODE_MFMA_FP8_X2) == MODE_MFMA_FP8_X2
-    assert hip.effective_mode(layer, 200, MODE_MFMA_FP8_X2) == MODE_MFMA_FP8
-    for cfg, act_mode in ((small, 2), (big, 1)):
+    for n, rows in ((20, 16), (200, 64)):
+        cfg = small.with_tokens(n)
+        assert hip.lib.ferrite_moe_layer_check(C.byref(layer.shape), n, MODE_MFMA_FP8_X2) == OK
+        assert hip.effective_mode(layer, n, MODE_MFMA_FP8_X2) == MODE_MFMA_FP8_X2
+        assert hip.unit_rows(layer, n, MODE_MFMA_FP8_X2) == rows
         x_np = synth.make_activations(cfg, seed=3)
-        out, v = run_layer(hip, layer, x_np, MODE_MFMA_FP8_X2)   # the same call for both batch sizes
-        import dataclasses
-        ref = oracle.moe_ffn_mxfp4(dataclasses.replace(inp, cfg=cfg, x=x_np), act_mode=act_mode, n_threads=8)
+        out, v = run_layer(hip, layer, x_np, MODE_MFMA_FP8_X2)
+        ref = oracle.moe_ffn_mxfp4(dataclasses.replace(inp, cfg=cfg, x=x_np), act_mode=2, n_threads=8)
         assert np.array_equal(v["ids"], ref["ids"].astype(np.int32))
-        assert max_abs_rel(out, ref["out"]) <= TOL_MFMA
-    # the fallen-back call is the one-term call, bit for bit
-    x_np = synth.make_activations(big, seed=3)
-    a, _ = run_layer(hip, layer, x_np, MODE_MFMA_FP8_X2)
-    b, _ = run_layer(hip, layer, x_np, MODE_MFMA_FP8)
-    assert np.array_equal(a, b)
+        assert max_abs_rel(out, ref["out"]) <= (TOL_MFMA_BF16_Y if rows == 64 else TOL_MFMA)
 
 
 @pytest.fixture
@@ -223,6 +234,37 @@ def test_prefill_main_loops_are_bit_identical(hip, overrides, n, hidden, inter, 
     finally:
         hip.set_override(OVERRIDE_PREFILL_TILE, 0)
         layer._ws.clear()
+
+
+@pytest.mark.parametrize("seed,n,hidden,inter,shared", [(6, 150, 256, 256, 128), (7, 700, 384, 256, 384),
+                                                        (8, 1100, 512, 128, 0), (9, 520, 4096, 1536, 1536)])
+def test_two_term_64_row_units_agree_with_16_row_units(hip, oracle, overrides, seed, n, hidden, inter, shared):
+    """Two-term activations on the tiled kernels (64-row units: both planes of a k step against the same weight
+    registers) and on the 16-row streaming kernels (a plane after the other per group of four k steps) add the same
+    products in a different order: f32 outputs agree to rounding, both sit within the MFMA bar of the two-term oracle
+    and inside 2e-2 of the f32 oracle, on ragged units and several units per expert."""
+    cfg = synth.MoeConfig(n, hidden, 8, 3, inter, shared, 4, 2)
+    inp = synth.make_inputs(cfg, seed=seed)
+    layer = hip.load_moe_layer(inp)
+    outs = {}
+    for rows, want in ((16, 16), (128, 64)):
+        overrides(unit_rows=rows, y_f32=1)
+        layer._ws.clear()
+        assert hip.unit_rows(layer, n, MODE_MFMA_FP8_X2) == want
+        outs[want], v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8_X2)
+    assert int(v["counts"].max()) > 64
+    ref = oracle.moe_ffn_mxfp4(inp, act_mode=2, n_threads=8)
+    ref32 = oracle.moe_ffn_mxfp4(inp, n_threads=8)
+    assert np.array_equal(v["ids"], ref["ids"].astype(np.int32))
+    assert max_abs_rel(outs[64], outs[16]) <= 1e-4
+    for o in outs.values():
+        assert max_abs_rel(o, ref["out"]) <= TOL_MFMA
+        assert max_abs_rel(o, ref32["out"]) <= TOL_X2_VS_F32
+    overrides(unit_rows=128, y_f32=0)
+    layer._ws.clear()
+    out_bf16, _ = run_layer(hip, layer, inp.x, MODE_MFMA_FP8_X2)
+    assert max_abs_rel(out_bf16, outs[64]) <= 2.0 ** -7
+    assert max_abs_rel(out_bf16, ref["out"]) <= TOL_MFMA_BF16_Y
 
 
 @pytest.mark.parametrize("variant", [0, 2])
@@ -425,9 +467,14 @@ def test_layer_error_paths(hip):
     xo = torch.from_numpy(odd.x).to(hip.device)
     oo = torch.empty_like(xo)
     hip.moe_layer_dev_mxfp4(ly, xo, oo, MODE_F32_CHECK)
-    with pytest.raises(FerriteError):
-        hip.moe_layer_dev_mxfp4(ly, xo, oo, MODE_MFMA_FP8)
+    # the library declines the MFMA mode for this shape (return code 2, nothing enqueued); the mirror falls back
+    import ctypes as C
+    from ferrite_amd.backend import DECLINED
+    assert hip.lib.ferrite_moe_layer_check(C.byref(ly.shape), 4, MODE_MFMA_FP8) == DECLINED
+    o2 = torch.empty_like(xo)
+    hip.moe_layer_dev_mxfp4(ly, xo, o2, MODE_MFMA_FP8)
     hip.sync()
+    assert torch.equal(oo, o2)
 
 
 def _block_case(cfg, seed):
@@ -539,7 +586,7 @@ def _scale_check(hip, oracle, cfg, n_sample, mode, seed=0, unit_tokens=False):
     counts = v["counts"]
     print(f"{cfg.name}: sample err {err:.3e} (vs f32 oracle {err32:.3e}); tokens/expert max {counts.max()} "
           f"mean {counts.mean():.1f}; experts hit {(counts > 0).sum()}")
-    assert err <= (TOL_MFMA_BF16_Y if hip.unit_rows(layer, cfg.n, mode) == 128 else TOL_MFMA)
+    assert err <= (TOL_MFMA_BF16_Y if hip.unit_rows(layer, cfg.n, mode) >= 64 else TOL_MFMA)
     assert err32 <= (TOL_X2_VS_F32 if mode == MODE_MFMA_FP8_X2 else TOL_X1_VS_F32)
     if unit_tokens:
         # Every row of one full unit and of the ragged last unit of one expert at this shape (evenly spaced tokens
@@ -557,16 +604,18 @@ def _scale_check(hip, oracle, cfg, n_sample, mode, seed=0, unit_tokens=False):
         err_u = max_abs_rel(out[toks], u["out"])
         print(f"{cfg.name}: expert {e} ({cnt} rows): all {rows} rows of its first unit and the {cnt % rows} rows of "
               f"its last one, {len(toks)} tokens: err {err_u:.3e}")
-        assert err_u <= (TOL_MFMA_BF16_Y if rows == 128 else TOL_MFMA)
+        assert err_u <= (TOL_MFMA_BF16_Y if rows >= 64 else TOL_MFMA)
     perm = np.random.default_rng(1).permutation(cfg.n)
     out_p, _ = run_layer(hip, layer, inp.x[perm], mode, bf16=cfg.act_bf16)
     assert np.array_equal(out_p, out[perm])
     return v
 
 
-def test_layer_c2_prefill_scale(hip, oracle):
-    """4096 tokens, ~256 tokens per expert."""
-    _scale_check(hip, oracle, synth.CONFIGS["c2"], n_sample=12, mode=MODE_MFMA_FP8, unit_tokens=True)
+@pytest.mark.parametrize("mode", [MODE_MFMA_FP8, MODE_MFMA_FP8_X2])
+def test_layer_c2_prefill_scale(hip, oracle, mode):
+    """4096 tokens, ~256 tokens per expert: one-term activations on 128-row units (the reference's serving format,
+    within 8e-2 of the f32 oracle) and two-term activations on 64-row units (within 2e-2 of it)."""
+    _scale_check(hip, oracle, synth.CONFIGS["c2"], n_sample=12, mode=mode, unit_tokens=True)
 
 
 @pytest.mark.parametrize("mode", [MODE_MFMA_FP8_X2, MODE_MFMA_FP8])
