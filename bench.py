@@ -138,7 +138,7 @@ def measured_traffic(config, kernel, build_id):
 
 
 def gate_up_roofline(cfg, n, unit_rows, gu_us, ab, config_name, build_id):
-    if unit_rows != 128:
+    if unit_rows < 64:
         # decode-sized batch: every weight byte is streamed once per unit; the kernel is HBM bound
         gbs = ab["gate_up"] / (gu_us * 1e-6) / 1e9
         r = {"bound": "hbm", "kernel": "gate_up_mfma_kernel", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
@@ -158,9 +158,10 @@ def gate_up_roofline(cfg, n, unit_rows, gu_us, ab, config_name, build_id):
     return r
 
 
-def f32_parity(oracle, inp, gpu_rows, ids_gpu, sel, n_threads):
+def f32_parity(oracle, inp, gpu_rows, ids_gpu, sel, n_threads, ref=None):
     """Distance of the GPU output rows `sel` from the f32 oracle (CpuBackend's arithmetic) on the same inputs."""
-    ref = oracle.moe_ffn_mxfp4(inp, act_mode=0, n_threads=n_threads, tok_sel=sel)
+    if ref is None:
+        ref = oracle.moe_ffn_mxfp4(inp, act_mode=0, n_threads=n_threads, tok_sel=sel)
     d = float(np.abs(gpu_rows.astype(np.float64) - ref["out"]).max() / np.abs(ref["out"]).max())
     return {"max_abs_rel": float(f"{d:.3e}"), "tokens": int(len(sel)),
             "router_ids_equal": bool(np.array_equal(ids_gpu, ref["ids"].astype(np.int32)))}
@@ -260,8 +261,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0,
                     help="chain this many distinct layers into one captured step (default: 42 for c4, else 1)")
     ap.add_argument("--mode", default="auto", choices=["auto", "fp8", "fp8x2"],
-                    help="activation format of the expert GEMMs: one e4m3 term, two (decode-sized batches; larger ones "
-                         "fall back to one), or auto = two where the library takes them")
+                    help="activation format of the expert GEMMs: one e4m3 term, two, or auto = two for decode-sized "
+                         "batches and one for prefill-sized ones")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-load-bench", action="store_true",
                     help="skip the checkpoint -> packed-buffer load measurement (writes a shard of the layer to TMPDIR)")
@@ -287,7 +288,16 @@ def main():
     hip = HipBackend()
     ev = HipEvents()
     n_layers = args.layers or (42 if args.config == "c4" else 1)
-    asked = MODE_MFMA_FP8 if args.mode == "fp8" else MODE_MFMA_FP8_X2   # auto: two terms where they are taken
+    asked = MODE_MFMA_FP8 if args.mode == "fp8" else MODE_MFMA_FP8_X2
+
+    def pick_mode(layer, n):
+        """auto: two terms for decode-sized batches (16-row units: the weight stream bounds the call and the second
+        term rides on it), the reference's one-term serving format for prefill-sized ones, whose two-term cost is
+        reported beside it; a mode the library declines falls back either way."""
+        want = asked
+        if args.mode == "auto" and hip.unit_rows(layer, n, MODE_MFMA_FP8_X2) != 16:
+            want = MODE_MFMA_FP8
+        return hip.effective_mode(layer, n, want)
     oracle = None
     if not args.no_cpu_baseline:
         from oracle import binding as oracle
@@ -303,7 +313,7 @@ def main():
     # ---- the chained decode step (configs[4]) as the workload of its own ----
     if n_layers > 1:
         step, layers, step_bytes = decode_step(hip, torch, synth, cfg, n_layers, asked, args.steps, args.warmup)
-        mode = hip.effective_mode(layers[0], n, asked)
+        mode = pick_mode(layers[0], n)
         inp = synth.make_inputs(cfg, seed=0)
         x = torch.from_numpy(inp.x).to(hip.device)
         x = x.to(torch.bfloat16) if cfg.act_bf16 else x
@@ -337,7 +347,7 @@ def main():
     inp = synth.make_inputs(cfg, seed=0)
     layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
     t_setup = time.time() - t0
-    mode = hip.effective_mode(layer, n, asked)   # the library declines two terms for prefill-sized batches
+    mode = pick_mode(layer, n)
     x = torch.from_numpy(inp.x).to(hip.device)
     if cfg.act_bf16:
         x = x.to(torch.bfloat16)
@@ -424,7 +434,7 @@ def main():
         pn = pcfg.n
         px_np = synth.make_activations(pcfg, seed=0)
         px = torch.from_numpy(px_np).to(hip.device).to(torch.bfloat16)
-        pmode = hip.effective_mode(layer, pn, asked)
+        pmode = pick_mode(layer, pn)
         pl = layer_leg(hip, torch, ev, layer, px, pn, pcfg, pmode, max(10, min(50, args.steps)), 20, stack=False)
         pcounts = pl["counts"]
         pab = algorithmic_bytes(pcfg, pn, int((pcounts > 0).sum()))
@@ -444,11 +454,24 @@ def main():
             import dataclasses
             sel = np.linspace(0, pn - 1, 32).astype(np.int32)
             pinp = dataclasses.replace(inp, cfg=pcfg, x=synth.round_to_bf16(px_np))
-            prefill["parity_vs_f32_oracle"] = f32_parity(oracle, pinp, pl["out"][sel], pl["ids"], sel, ncores)
+            pref = oracle.moe_ffn_mxfp4(pinp, act_mode=0, n_threads=ncores, tok_sel=sel)
+            prefill["parity_vs_f32_oracle"] = f32_parity(oracle, pinp, pl["out"][sel], pl["ids"], sel, ncores, pref)
             prefill["parity_vs_f32_oracle"]["what"] = ("one e4m3 term per activation (three mantissa bits) against the "
                                                        "unquantised f32 oracle; router ids compared for all tokens")
             del pinp
-        del px, pl
+        # the same chunk with two e4m3 terms per activation (64-row units): what the 2e-2 bar costs at prefill
+        from ferrite_amd.backend import MODE_MFMA_FP8_X2 as _X2
+        pl2 = layer_leg(hip, torch, ev, layer, px, pn, pcfg, _X2, max(10, min(30, args.steps)), 10, stack=False)
+        prefill["two_term"] = {"activation_terms": pl2["terms"], "unit_rows": hip.unit_rows(layer, pn, _X2),
+                               "us_per_layer": round(pl2["us"], 2),
+                               "tokens_per_s": round(pn / (pl2["us"] * 1e-6), 1),
+                               "stage_us": {k: round(v, 2) for k, v in pl2["stage_us"].items()},
+                               "gate_up_kernel_us": round(pl2["gu_us"], 2),
+                               "what": "both planes of x and of the SwiGLU output, a second MFMA per tile against the "
+                                       "same weight registers: twice the MFMAs and fills of the one-term chunk"}
+        if oracle is not None:
+            prefill["two_term"]["parity_vs_f32_oracle"] = f32_parity(oracle, None, pl2["out"][sel], pl2["ids"], sel, ncores, pref)
+        del px, pl, pl2
 
     # the row before the layer: one layer's shard (safetensors, the reference's tensor names) streamed from the
     # page cache into the packed buffer; PCIe-bound, priced against a pinned -> device copy of the same size
