@@ -555,7 +555,8 @@ class HipBackend:
         return layer._ws[key]
 
     def unit_rows(self, layer: MoeLayer, n: int, mode: int = MODE_MFMA_FP8) -> int:
-        """Token tile of the expert GEMMs for such a call: 16 (streaming kernels) or 128 (LDS-tiled kernels)."""
+        """Token tile of the expert GEMMs for such a call: 16 (streaming kernels), or the tiled kernels' 128 (one-term
+        activations) / 64 (two-term)."""
         return int(self.lib.ferrite_moe_layer_unit_rows(C.byref(layer.shape), n, self.effective_mode(layer, n, mode)))
 
     def moe_layer_dev_mxfp4(self, layer: MoeLayer, x: torch.Tensor, out: torch.Tensor, mode: int = MODE_MFMA_FP8,

@@ -36,11 +36,11 @@ inline int max_units_for(int n, int topk, int n_experts, int has_shared, int uni
     return (int)u;
 }
 
-// Rows per unit for a layer call: 128-row units (both GEMM operands tiled through LDS) once the average expert
-// sees enough rows to fill them, 16-row units (weights streamed once per unit) below that.  A process-wide override
-// (ferrite_hip_set_override, a test hook) forces either; nothing here reads the environment.
+// Rows per unit for a layer call: the tiled kernels (units of 128 rows, 64 with two-term activations) once the
+// average expert sees enough rows to fill them, 16-row units (weights streamed once per unit) below that.  A
+// process-wide override (ferrite_hip_set_override, a test hook) forces either; nothing here reads the environment.
 int unit_rows_for(int n, int topk, int n_experts, bool two_term);
-// Element type of the expert outputs `y` in the workspace: bf16 for 128-row units (prefill-sized batches, where the
+// Element type of the expert outputs `y` in the workspace: bf16 for the tiled kernels (prefill-sized batches, where the
 // y round trip through HBM is a tenth of the layer), f32 otherwise.  The FERRITE_OVERRIDE_Y_F32 override forces f32.
 int y_dtype_for(int unit_rows);
 

@@ -43,9 +43,10 @@ extern "C" {
 #define FERRITE_MODE_MFMA_FP8 1    /* activations quantised e4m3 per 32 (e8m0 scale), block-scaled MFMA */
 #define FERRITE_MODE_MFMA_FP8_X2 2 /* the same with two-term activations: x ~ q1*s1 + q2*s2, the second term being the
                                     * e4m3-per-32 quantisation of what the first leaves over (about 8 significant
-                                    * bits, bf16-class).  Decode-sized batches only (n*topk < 48*n_experts), where
-                                    * the matrix cores idle behind the weight stream and the second term is free;
-                                    * larger batches return FERRITE_DECLINED (use FERRITE_MODE_MFMA_FP8). */
+                                    * bits, bf16-class).  For decode-sized batches (n*topk < 48*n_experts) the
+                                    * matrix cores idle behind the weight stream and the second term is nearly free;
+                                    * prefill-sized batches are bound by the matrix cores and pay for it (64-row
+                                    * units, twice the MFMAs per row: about 1.6 times the one-term layer). */
 
 typedef void* ferrite_stream_t;
 
@@ -63,8 +64,9 @@ int ferrite_hip_warmup(void);
 /* Process-wide test hooks (the reference's counterparts are environment gates read once into a OnceLock,
  * cuda.rs:5730-5731; here nothing reads the environment).  They change how a layer call tiles its work, and with it
  * the workspace layout: set them before sizing a workspace, not between sizing and use.
- *   FERRITE_OVERRIDE_UNIT_ROWS  0 = automatic (default), 16 or 128 = force that token tile for the expert GEMMs
- *   FERRITE_OVERRIDE_Y_F32      1 = keep the expert outputs `y` in f32 on the 128-row path (default 0: bf16)
+ *   FERRITE_OVERRIDE_UNIT_ROWS  0 = automatic (default), 16 = force the 16-row streaming kernels, 128 = force the
+ *                               tiled kernels (units of 128 rows, or of 64 rows with two-term activations)
+ *   FERRITE_OVERRIDE_Y_F32      1 = keep the expert outputs `y` in f32 on the tiled path (default 0: bf16)
  *   FERRITE_OVERRIDE_PREFILL_TILE  main loop of the 128-row units: 0 = default (gate/up: weights streamed into
  *                               registers by blocks of 8 waves; down: both operands staged through LDS), 1 = staged
  *                               for both GEMMs, 2 / 3 = streamed by blocks of 8 / 4 waves for both (same bits)
@@ -204,20 +206,20 @@ typedef struct ferrite_moe_workspace_view {
     int32_t* active;     /* [E] */
     int32_t* n_active;   /* [1] */
     float* y;            /* [(n*topk + n), H] expert outputs in grouped order, then the shared expert's rows; f32,
-                          * except bf16 (same shape, half the bytes) when ferrite_moe_layer_unit_rows() is 128 and
-                          * the FERRITE_OVERRIDE_Y_F32 override is off */
+                          * except bf16 (same shape, half the bytes) when ferrite_moe_layer_unit_rows() is 64 or
+                          * 128 and the FERRITE_OVERRIDE_Y_F32 override is off */
 } ferrite_moe_workspace_view;
 
 /* What a layer call with these arguments would answer before it enqueues anything: FERRITE_OK, or
  * FERRITE_DECLINED (this batch size / shape is outside this mode's contract: the caller falls back to another mode,
- * as CudaBackend does when a fused kernel declines, cuda.rs:5763-5765,5940,5990 - in particular
- * FERRITE_MODE_MFMA_FP8_X2 declines prefill-sized batches, whose fallback is FERRITE_MODE_MFMA_FP8), or
+ * as CudaBackend does when a fused kernel declines, cuda.rs:5763-5765,5940,5990 - the order is two-term MFMA,
+ * one-term MFMA, f32; the MFMA modes decline hidden / intermediate sizes that are not multiples of 128), or
  * FERRITE_ERR_INVALID_ARG.  A declined mode has no workspace size either (ferrite_moe_layer_workspace_bytes is 0). */
 int ferrite_moe_layer_check(const ferrite_moe_shape* shape, int n, int mode);
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
 /* Rows per unit (the token tile of the expert GEMMs) a layer call with these arguments uses: 16 = weights streamed
- * once per unit (decode-sized batches, any activation format),
- * 128 = both operands tiled through LDS (prefill-sized batches); 0 for an
+ * once per unit (decode-sized batches, any activation format); for prefill-sized batches the tiled kernels,
+ * 128 = one-term activations, 64 = two-term activations (both planes of 64 rows fill the same tile); 0 for an
  * unsupported shape.  The choice is a pure function of (shape, n, mode) and of the FERRITE_OVERRIDE_UNIT_ROWS
  * override, like the workspace layout that depends on it.
  * No counterpart in the reference, whose grouped GEMM has one tile shape (dsv41_moe.cu); informational. */
