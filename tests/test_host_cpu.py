@@ -101,6 +101,38 @@ def test_overrides_validate_their_arguments():
     assert lib.ferrite_moe_layer_unit_rows(C.byref(shape), 32, backend.MODE_MFMA_FP8) == 16
 
 
+def test_layer_check_answers_without_a_gpu_and_units_follow_mode_and_size():
+    """ferrite_moe_layer_check is host arithmetic: what a layer call would answer before it enqueues anything.  The
+    MFMA modes decline sizes that are not multiples of 128 (the f32 mode takes them: the order the host mirrors fall
+    back in); two-term activations are served at every batch size, on 16-row units for decode-sized batches and on
+    64-row units (128 with one term) for prefill-sized ones; a declined call has no workspace size."""
+    from ferrite_amd import backend
+    lib = backend.load_library()
+    shape = backend.MoeShape(4096, 128, 8, 1536, 1536, 8, 4, 2.5, 10.0)
+    for n in (32, 192, 4096):
+        for mode in (backend.MODE_F32_CHECK, backend.MODE_MFMA_FP8, backend.MODE_MFMA_FP8_X2):
+            assert lib.ferrite_moe_layer_check(C.byref(shape), n, mode) == backend.OK
+    rows = lambda n, mode: lib.ferrite_moe_layer_unit_rows(C.byref(shape), n, mode)
+    assert [rows(n, backend.MODE_MFMA_FP8) for n in (32, 192, 767, 768, 4096)] == [16, 16, 16, 128, 128]
+    assert [rows(n, backend.MODE_MFMA_FP8_X2) for n in (32, 192, 767, 768, 4096)] == [16, 16, 16, 64, 64]
+    assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 128) == backend.OK
+    assert rows(32, backend.MODE_MFMA_FP8_X2) == 64 and rows(32, backend.MODE_MFMA_FP8) == 128
+    assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 16) == backend.OK
+    assert rows(4096, backend.MODE_MFMA_FP8_X2) == 16
+    assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 0) == backend.OK
+    sz = lambda n, mode: lib.ferrite_moe_layer_workspace_bytes(C.byref(shape), n, mode)
+    assert sz(4096, backend.MODE_MFMA_FP8_X2) > sz(4096, backend.MODE_MFMA_FP8) > 0      # the second planes
+    odd = backend.MoeShape(160, 8, 3, 96, 64, 4, 2, 2.5, 10.0)
+    for n in (20, 200):
+        assert lib.ferrite_moe_layer_check(C.byref(odd), n, backend.MODE_MFMA_FP8_X2) == backend.DECLINED
+        assert lib.ferrite_moe_layer_check(C.byref(odd), n, backend.MODE_MFMA_FP8) == backend.DECLINED
+        assert lib.ferrite_moe_layer_check(C.byref(odd), n, backend.MODE_F32_CHECK) == backend.OK
+        assert sz(n, backend.MODE_MFMA_FP8) > 0
+        assert lib.ferrite_moe_layer_workspace_bytes(C.byref(odd), n, backend.MODE_MFMA_FP8) == 0
+    assert lib.ferrite_moe_layer_check(C.byref(shape), 32, 9) == backend.ERR_INVALID_ARG
+    assert lib.ferrite_moe_layer_check(None, 32, backend.MODE_MFMA_FP8) == backend.ERR_INVALID_ARG
+
+
 def test_library_sources_read_no_environment():
     """Launchers may be recorded into a stream capture; the reference reads its gates once for that reason
     (cuda.rs:5730-5731).  Here no source of the library reads the environment at all."""
