@@ -337,6 +337,30 @@ struct PermArgs {
     int unit_cap, max_units, has_shared;
 };
 
+// How an expert's c rows are cut into `units` = ceil(c / cap) units.  With 16-row units the cut is every cap rows.
+// The tiled kernels' units are balanced in whole 16-row tiles instead (the first `rem` units hold one tile more than
+// the others): the blocks that work on the units of one expert then run at the same pace and fetch the expert's
+// weights together, where a nearly empty last unit runs ahead of the full ones and both miss L2.
+struct UnitCut {
+    int c, cap, base, rem;   // base, rem: tiles per unit and units with one more (tiled kernels only)
+    __device__ __forceinline__ UnitCut(int c_, int cap_, int units) : c(c_), cap(cap_), base(0), rem(0) {
+        if (cap > 16 && units > 0) {
+            const int tiles = (c + 15) >> 4;
+            base = tiles / units;
+            rem = tiles - base * units;
+        }
+    }
+    __device__ __forceinline__ void span(int i, int& r0, int& rows) const {
+        if (cap <= 16) {
+            r0 = i * cap;
+            rows = min(cap, c - r0);
+        } else {
+            r0 = (i * base + min(i, rem)) * 16;
+            rows = min(c, r0 + (base + (i < rem ? 1 : 0)) * 16) - r0;
+        }
+    }
+};
+
 // wave 0 of a block: exclusive scan over experts + active list + unit tables. cnt[] readable by the wave.
 __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t* starts_lds) {
     const int lane = threadIdx.x & 63;
@@ -373,11 +397,14 @@ __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t*
             ract += c > 0;
             if (a.unit_cap > 0) {
                 const int first = rtile, cnt_e = (c + a.unit_cap - 1) / a.unit_cap;
-                for (int r = 0; r < c; r += a.unit_cap) {
+                const UnitCut cut(c, a.unit_cap, cnt_e);
+                for (int i2 = 0; i2 < cnt_e; ++i2) {
                     if (rtile < a.max_units) {
+                        int r0, rows;
+                        cut.span(i2, r0, rows);
                         a.unit_expert[rtile] = e;
-                        a.unit_row0[rtile] = run + r;
-                        a.unit_rows[rtile] = min(a.unit_cap, c - r);
+                        a.unit_row0[rtile] = run + r0;
+                        a.unit_rows[rtile] = rows;
                         if (a.unit_first) { a.unit_first[rtile] = first; a.unit_count[rtile] = cnt_e; }
                     }
                     ++rtile;
@@ -396,12 +423,15 @@ __device__ void perm_expert_scan(const PermArgs& a, const int32_t* cnt, int32_t*
     if (a.unit_cap > 0) {
         // shared expert: all n tokens, rows [n*topk, n*topk + n) of the activation / output row space
         int sh_tiles = a.has_shared ? (a.n + a.unit_cap - 1) / a.unit_cap : 0;
+        const UnitCut sh_cut(a.n, a.unit_cap, sh_tiles);
         for (int i = lane; i < sh_tiles; i += 64) {
             int u = total_tile + i;
             if (u < a.max_units) {
+                int r0, rows;
+                sh_cut.span(i, r0, rows);
                 a.unit_expert[u] = E;
-                a.unit_row0[u] = a.n * a.topk + i * a.unit_cap;
-                a.unit_rows[u] = min(a.unit_cap, a.n - i * a.unit_cap);
+                a.unit_row0[u] = a.n * a.topk + r0;
+                a.unit_rows[u] = rows;
                 if (a.unit_first) { a.unit_first[u] = total_tile; a.unit_count[u] = sh_tiles; }
             }
         }

@@ -594,21 +594,26 @@ def _scale_check(hip, oracle, cfg, n_sample, mode, seed=0, unit_tokens=False):
     assert err <= (TOL_MFMA_BF16_Y if hip.unit_rows(layer, cfg.n, mode) >= 64 else TOL_MFMA)
     assert err32 <= (TOL_X2_VS_F32 if mode == MODE_MFMA_FP8_X2 else TOL_X1_VS_F32)
     if unit_tokens:
-        # Every row of one full unit and of the ragged last unit of one expert at this shape (evenly spaced tokens
-        # touch a unit's first rows at best): the expert whose row count leaves the shortest non-empty last unit
-        # among those with at least one full unit.
+        # Every row of the first and of the last unit of one expert at this shape (evenly spaced tokens touch a
+        # unit's first rows at best).  The tiled kernels cut an expert's rows into ceil(rows / cap) units balanced in
+        # whole 16-row tiles (the first units hold one tile more): take the expert with several units whose last
+        # unit ends in the emptiest ragged tile.
         rows = hip.unit_rows(layer, cfg.n, mode)
-        cand = [e for e in range(cfg.n_experts) if counts[e] > rows and counts[e] % rows]
-        e = min(cand, key=lambda i: counts[i] % rows)
+        cand = [e for e in range(cfg.n_experts) if counts[e] > rows and counts[e] % 16]
+        e = min(cand, key=lambda i: counts[i] % 16)
         start, cnt = int(v["starts"][e]), int(counts[e])
-        last0 = start + (cnt // rows) * rows
-        grouped = np.concatenate([np.arange(start, start + rows), np.arange(last0, start + cnt)])
+        units, tiles = -(-cnt // rows), -(-cnt // 16)
+        base, rem = divmod(tiles, units)
+        first_rows = (base + (1 if rem else 0)) * 16
+        last0 = ((units - 1) * base + min(units - 1, rem)) * 16
+        assert first_rows <= rows and 0 < cnt - last0 <= rows
+        grouped = np.concatenate([np.arange(start, start + first_rows), np.arange(start + last0, start + cnt)])
         toks = np.unique(v["gather_src"][grouped] // cfg.topk).astype(np.int32)
         assert len(toks) == len(grouped)   # an expert holds a token once
         u = oracle.moe_ffn_mxfp4(inp, act_mode=ACT_MODE[mode], n_threads=16, tok_sel=toks)
         err_u = max_abs_rel(out[toks], u["out"])
-        print(f"{cfg.name}: expert {e} ({cnt} rows): all {rows} rows of its first unit and the {cnt % rows} rows of "
-              f"its last one, {len(toks)} tokens: err {err_u:.3e}")
+        print(f"{cfg.name}: expert {e} ({cnt} rows in {units} units): all {first_rows} rows of its first unit and the "
+              f"{cnt - last0} rows of its last one, {len(toks)} tokens: err {err_u:.3e}")
         assert err_u <= (TOL_MFMA_BF16_Y if rows >= 64 else TOL_MFMA)
     perm = np.random.default_rng(1).permutation(cfg.n)
     out_p, _ = run_layer(hip, layer, inp.x[perm], mode, bf16=cfg.act_bf16)
