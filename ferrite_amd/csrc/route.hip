@@ -1136,12 +1136,9 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const XT* __restrict__
     }
 }
 
-template <typename XT>
-static int launch_router_tile(const void* x, const float* router_t, int n, int H, int E, float* logits, hipStream_t st) {
-    const int Epad = (E + 63) / 64 * 64;
-    const XT* xp = static_cast<const XT*>(x);
-    const float4* wp = reinterpret_cast<const float4*>(router_t);
-    constexpr int T = 4;
+template <typename XT, int T>
+static int launch_router_tile_t(const XT* xp, const float4* wp, int n, int H, int E, int Epad, float* logits,
+                                hipStream_t st) {
     dim3 grid(1, (n + 4 * T - 1) / (4 * T));
     // two expert blocks per wave halve the weight traffic, but only when enough waves remain to hide latency
     if (Epad % 128 == 0 && (long)(Epad / 128) * grid.y * 4 >= 4096) {
@@ -1152,6 +1149,20 @@ static int launch_router_tile(const void* x, const float* router_t, int n, int H
         router_tile_kernel<XT, T, 1><<<grid, 256, 0, st>>>(xp, wp, n, H, E, Epad, logits);
     }
     return check_launch("router_tile");
+}
+
+// Tokens per wave: four share a wave's weight loads, but a wave walks its chains one after the other, so with few
+// tokens the kernel's time is the length of one wave's work (320 tokens x 128 experts at four tokens per wave are
+// 160 waves on 1024 SIMDs: 114 us).  Fewer tokens per wave while that leaves SIMDs idle.
+template <typename XT>
+static int launch_router_tile(const void* x, const float* router_t, int n, int H, int E, float* logits, hipStream_t st) {
+    const int Epad = (E + 63) / 64 * 64;
+    const XT* xp = static_cast<const XT*>(x);
+    const float4* wp = reinterpret_cast<const float4*>(router_t);
+    const long groups = Epad / 64;
+    if (groups * ((n + 3) / 4) >= 1024) return launch_router_tile_t<XT, 4>(xp, wp, n, H, E, Epad, logits, st);
+    if (groups * ((n + 1) / 2) >= 1024) return launch_router_tile_t<XT, 2>(xp, wp, n, H, E, Epad, logits, st);
+    return launch_router_tile_t<XT, 1>(xp, wp, n, H, E, Epad, logits, st);
 }
 
 // Router GEMM alone from the transposed weight (any n): logits only.

@@ -43,7 +43,7 @@ extern "C" {
 #define FERRITE_MODE_MFMA_FP8 1    /* activations quantised e4m3 per 32 (e8m0 scale), block-scaled MFMA */
 #define FERRITE_MODE_MFMA_FP8_X2 2 /* the same with two-term activations: x ~ q1*s1 + q2*s2, the second term being the
                                     * e4m3-per-32 quantisation of what the first leaves over (about 8 significant
-                                    * bits, bf16-class).  For decode-sized batches (n*topk < 48*n_experts) the
+                                    * bits, bf16-class).  For decode-sized batches (n*topk < 16*n_experts) the
                                     * matrix cores idle behind the weight stream and the second term is nearly free;
                                     * prefill-sized batches are bound by the matrix cores and pay for it (64-row
                                     * units, twice the MFMAs per row: about 1.6 times the one-term layer). */
@@ -218,7 +218,7 @@ typedef struct ferrite_moe_workspace_view {
 int ferrite_moe_layer_check(const ferrite_moe_shape* shape, int n, int mode);
 size_t ferrite_moe_layer_workspace_bytes(const ferrite_moe_shape* shape, int n, int mode);
 /* Rows per unit (the token tile of the expert GEMMs) a layer call with these arguments uses: 16 = weights streamed
- * once per unit (decode-sized batches, any activation format); for prefill-sized batches the tiled kernels,
+ * once per unit (decode-sized batches: n*topk < 16*n_experts, any activation format); beyond that the tiled kernels,
  * 128 = one-term activations, 64 = two-term activations (both planes of 64 rows fill the same tile); 0 for an
  * unsupported shape.  The choice is a pure function of (shape, n, mode) and of the FERRITE_OVERRIDE_UNIT_ROWS
  * override, like the workspace layout that depends on it.

@@ -113,8 +113,8 @@ def test_layer_check_answers_without_a_gpu_and_units_follow_mode_and_size():
         for mode in (backend.MODE_F32_CHECK, backend.MODE_MFMA_FP8, backend.MODE_MFMA_FP8_X2):
             assert lib.ferrite_moe_layer_check(C.byref(shape), n, mode) == backend.OK
     rows = lambda n, mode: lib.ferrite_moe_layer_unit_rows(C.byref(shape), n, mode)
-    assert [rows(n, backend.MODE_MFMA_FP8) for n in (32, 192, 767, 768, 4096)] == [16, 16, 16, 128, 128]
-    assert [rows(n, backend.MODE_MFMA_FP8_X2) for n in (32, 192, 767, 768, 4096)] == [16, 16, 16, 64, 64]
+    assert [rows(n, backend.MODE_MFMA_FP8) for n in (32, 192, 255, 256, 4096)] == [16, 16, 16, 128, 128]
+    assert [rows(n, backend.MODE_MFMA_FP8_X2) for n in (32, 192, 255, 256, 4096)] == [16, 16, 16, 64, 64]
     assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 128) == backend.OK
     assert rows(32, backend.MODE_MFMA_FP8_X2) == 64 and rows(32, backend.MODE_MFMA_FP8) == 128
     assert lib.ferrite_hip_set_override(backend.OVERRIDE_UNIT_ROWS, 16) == backend.OK
