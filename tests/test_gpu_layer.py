@@ -391,14 +391,80 @@ def test_chained_layers_in_one_graph(hip, oracle, mode):
     hip.graph_destroy(trace)
 
 
-@pytest.mark.parametrize("n_experts,modes", [(16, (MODE_MFMA_FP8,)), (64, (MODE_MFMA_FP8, MODE_MFMA_FP8_X2))])
-def test_layer_unfused_head_path(hip, oracle, n_experts, modes):
+def test_decode_step_chain_at_the_benchmark_shape(hip, oracle):
+    """Three layers of the 42-layer decode step at its real shape (192 tokens, H 4096, 128 experts, I 1536, two-term
+    activations): every layer has its own weights, normalises the previous layer's output and runs on it (the block
+    call without hc_post), all on one workspace in one graph.  Every layer's output is compared with the oracle's
+    rmsnorm -> layer on the input that layer saw (routing bit-exact), and a replay of the graph on fresh input equals
+    the eager chain bit for bit."""
+    import dataclasses
+    cfg, n_layers = synth.CONFIGS["c4"], 3
+    n, mode = cfg.n, MODE_MFMA_FP8_X2
+    inps = [synth.make_inputs(cfg, seed=0, layer=l) for l in range(n_layers)]
+    layers = [hip.load_moe_layer(i, keep_checkpoint_layout=False) for i in inps]
+    g = torch.Generator(device="cpu").manual_seed(2)
+    norm_ws = [(torch.rand(cfg.hidden, generator=g) + 0.5) for _ in layers]
+    norm_d = [w.to(hip.device) for w in norm_ws]
+    bws = hip.block_workspace(layers[0], n, mode)
+    assert hip.unit_rows(layers[0], n, mode) == 16
+    x_static = torch.zeros(n, cfg.hidden, device=hip.device)
+
+    def chain(src, outs):
+        for l, ly in enumerate(layers):
+            hip.moe_block_mxfp4(ly, src, norm_d[l], 1e-6, None, None, None, outs[l], mode, workspace=bws)
+            src = outs[l]
+
+    x0 = torch.from_numpy(synth.round_to_bf16(inps[0].x)).to(hip.device)
+    eager = [torch.empty(n, cfg.hidden, device=hip.device) for _ in layers]
+    chain(x0, eager)
+    hip.sync()
+    src = x0
+    for l in range(n_layers):
+        x_in = src.cpu().numpy()
+        hfn = oracle.rmsnorm(x_in, norm_ws[l].numpy(), 1e-6)
+        ref = oracle.moe_ffn_mxfp4(dataclasses.replace(inps[l], x=hfn), act_mode=2, n_threads=16)
+        ref32 = oracle.moe_ffn_mxfp4(dataclasses.replace(inps[l], x=hfn), act_mode=0, n_threads=16)
+        got = eager[l].cpu().numpy()
+        err, err32 = max_abs_rel(got, ref["out"]), max_abs_rel(got, ref32["out"])
+        print(f"decode-step chain, layer {l}: vs two-term oracle {err:.3e}, vs f32 oracle {err32:.3e}")
+        assert err <= TOL_MFMA and err32 <= TOL_X2_VS_F32
+        src = eager[l]
+    # the routing tables the last layer left in the shared workspace are the oracle's for the input it saw
+    v = {k: t.cpu().numpy() for k, t in hip.workspace_view(layers[-1], n, mode, workspace=bws).items() if k != "y"}
+    check_routing(v, ref32, oracle, cfg)
+    staged = [torch.empty(n, cfg.hidden, device=hip.device) for _ in layers]
+    chain(x_static, staged)
+    hip.sync()
+    hip.begin_capture()
+    chain(x_static, staged)
+    trace = hip.end_capture()
+    assert [r.op for r in trace.ops] == ["moe_block_mxfp4"] * n_layers
+    for seed in (41, 42):
+        x = torch.from_numpy(synth.round_to_bf16(synth.random_normal(seed, 1, n * cfg.hidden).reshape(n, cfg.hidden)))
+        x = x.to(hip.device)
+        chain(x, eager)
+        hip.sync()
+        x_static.copy_(x)
+        torch.cuda.synchronize()
+        hip.begin_verify(trace)
+        assert hip.end_verify()
+        for l in range(n_layers):
+            assert torch.equal(staged[l], eager[l])
+    hip.graph_destroy(trace)
+
+
+@pytest.mark.parametrize("n_experts,rows", [(16, 128), (64, 128), (128, 16)])
+def test_layer_unfused_head_path(hip, oracle, n_experts, rows):
     """More tokens than the fused routing kernel takes (n > 256): separate router GEMM, routing, three-phase
-    permutation and quantisation launches; results must not depend on which head ran.  With 16 experts the batch is
-    prefill-sized (128-row units, one-term only), with 64 it still streams the weights (16- / 8-row units)."""
+    permutation and quantisation launches; results must not depend on which head ran.  With 16 and 64 experts the
+    average expert sees 16 rows or more (the tiled kernels: 128-row units, 64 with two terms), with 128 it still
+    streams the weights (16-row units); both activation formats in each."""
+    modes = (MODE_MFMA_FP8, MODE_MFMA_FP8_X2)
     cfg = synth.MoeConfig(300, 256, n_experts, 4, 128, 128, 4, 2)
     inp = synth.make_inputs(cfg, seed=9)
     layer = hip.load_moe_layer(inp)
+    assert hip.unit_rows(layer, 300, MODE_MFMA_FP8) == rows
+    assert hip.unit_rows(layer, 300, MODE_MFMA_FP8_X2) == min(rows, 64)
     ref32 = oracle.moe_ffn_mxfp4(inp, n_threads=8)
     out, v = run_layer(hip, layer, inp.x, MODE_F32_CHECK)
     check_routing(v, ref32, oracle, cfg)
