@@ -4,14 +4,20 @@
 One "step" = one pass of the fused layer (router GEMM -> routing -> permutation -> activation quantisation ->
 gate/up GEMM + SwiGLU -> down GEMM -> combine) over one batch of synthetic tokens, replayed from a captured
 hipGraph the way a decode step runs in production.  Inputs and weights are resident in HBM before the timed
-region.  Prints ONE JSON line (see README / DESIGN for the fields).
+region.  Prints ONE JSON line: metric / value (tokens per second of the layer) / ms_per_step and the workload in
+"config"; "roofline" for the gate/up kernel (algorithmic bytes or flops per launch over its duration, measured with
+HIP events on the launch stream; "traffic" = counter-derived HBM bytes per launch of the profiled build);
+"cpu_baseline" (the CPU oracle on the same tokens); and the legs described below.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--no-cpu-baseline]
 
-The default run times the decode layer (c1: 32 tokens) and, on the same weights, a bounded prefill leg (c2: 4096
-tokens) reported under "prefill".  --config c4 runs the 42-layer decode step: every layer has its own weights, the
-layers are chained (rmsnorm of a layer's output is the next layer's input) and share one workspace, and the whole
-step is one hipGraph.
+The default run times the decode layer (c1: 32 tokens, two-term activations; "decode_fp8": the same with one term)
+and, on the same weights, a bounded prefill leg (c2: 4096 tokens, one-term activations, with its own roofline and
+distance to the f32 oracle, and "two_term": the same chunk with two-term activations) reported under "prefill";
+"decode_step" is the 42-layer decode step (c4: 192 tokens): every layer has its own weights, the layers are chained
+(rmsnorm of a layer's output is the next layer's input) and share one workspace, and the whole step is one
+hipGraph (--config c4 times that step alone).  "block_rmsnorm_layer_hc_post" and "checkpoint_load" time the steps
+either side of the layer.
 """
 from __future__ import annotations
 
