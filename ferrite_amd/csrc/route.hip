@@ -1017,8 +1017,12 @@ static int warmup_head() {
     return LdsLimit<&moe_head_kernel<XT, kFused, 2, 32>>::ensure(cap);
 }
 
+template <typename XT> __global__ void router_lds_kernel(const XT*, const float4*, int, int, int, int, float*);
+
 int warmup_route() {
     int rc;
+    if ((rc = LdsLimit<&router_lds_kernel<float>>::ensure(70 * 1024))) return rc;
+    if ((rc = LdsLimit<&router_lds_kernel<uint16_t>>::ensure(70 * 1024))) return rc;
     if ((rc = warmup_head<float, true>())) return rc;
     if ((rc = warmup_head<uint16_t, true>())) return rc;
     if ((rc = warmup_head<float, false>())) return rc;
@@ -1136,6 +1140,86 @@ __global__ __launch_bounds__(256) void router_tile_kernel(const XT* __restrict__
     }
 }
 
+// The same chain for batches of a few hundred tokens, where the kernel above leaves SIMDs idle (four tokens per
+// wave: 160 waves at 320 tokens x 128 experts, 115 us) or, with one token per wave, pulls every wave's own copy of
+// the router weights through the vector memory path (1 KiB per wave and four k: 79 us, bound by the 64 bytes per
+// clock a CU's address unit handles).  Here the four waves of a block work on four tokens against the same 64
+// experts and share the weights through LDS: a chunk of RL_KC k (all 64 experts) is fetched once per block into a
+// two-slot ring, a chunk ahead of its use, each wave stages its own token's activations (as f32) beside it, and a
+// lane reads its expert's float4 and the token's float4 (a broadcast) per four k.  One barrier per chunk.
+typedef float rl_f4 __attribute__((ext_vector_type(4)));
+constexpr int RL_KC = 128;                                   // k per chunk
+constexpr int RL_W_SLOT = RL_KC / 4 * 64;                    // float4 of weights per slot (32 KiB)
+constexpr int RL_X_SLOT = 4 * RL_KC / 4;                     // float4 of activations per slot: 4 tokens x RL_KC f32
+constexpr size_t RL_LDS_BYTES = 2 * (size_t)(RL_W_SLOT + RL_X_SLOT) * 16;
+
+// A thread's share of chunk c: weight rows wave + 4 i of the chunk for expert e0 + lane, and two activations of the
+// wave's token.
+template <typename XT>
+__device__ __forceinline__ void rl_fetch(rl_f4 (&wr)[RL_KC / 16], float (&xv)[2], const rl_f4* __restrict__ wt,
+                                         const XT* __restrict__ xrow, int Epad, int col, int wave, int lane, int c) {
+    const rl_f4* src = wt + (size_t)(c * (RL_KC / 4) + wave) * Epad + col;
+#pragma unroll
+    for (int i = 0; i < RL_KC / 16; ++i) wr[i] = src[(size_t)(4 * i) * Epad];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const XT v = xrow[c * RL_KC + i * 64 + lane];
+        if constexpr (sizeof(XT) == 4) xv[i] = v; else xv[i] = u2f((uint32_t)v << 16);
+    }
+}
+
+__device__ __forceinline__ void rl_stash(rl_f4* slot, const rl_f4 (&wr)[RL_KC / 16], const float (&xv)[2], int wave,
+                                         int lane) {
+#pragma unroll
+    for (int i = 0; i < RL_KC / 16; ++i) slot[(wave + 4 * i) * 64 + lane] = wr[i];
+    float* xs = reinterpret_cast<float*>(slot + RL_W_SLOT) + wave * RL_KC;
+    xs[lane] = xv[0];
+    xs[64 + lane] = xv[1];
+}
+
+template <typename XT>
+__global__ __launch_bounds__(256) void router_lds_kernel(const XT* __restrict__ x, const float4* __restrict__ wt,
+                                                         int n, int H, int E, int Epad, float* __restrict__ logits) {
+    extern __shared__ __align__(16) unsigned char rl_raw[];
+    rl_f4* lds = reinterpret_cast<rl_f4*>(rl_raw);
+    const rl_f4* wt4 = reinterpret_cast<const rl_f4*>(wt);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t = blockIdx.y * 4 + wave;
+    const int col = blockIdx.x * 64 + lane;
+    const XT* xrow = x + (size_t)min(t, n - 1) * H;
+    const int nchunk = H / RL_KC;
+    // One register set: chunk c + 1 is in flight while chunk c is walked.  (Two sets, a chunk fetched two chunk
+    // times ahead, measured slower: 67 against 48 us at 320 tokens.  What bounds a block is LDS bandwidth - 160 KiB
+    // of reads and writes per chunk - and the chains' own instructions, one after the other in a lone wave.)
+    rl_f4 wr[RL_KC / 16];
+    float xv[2];
+    float acc = 0.0f;
+    rl_fetch(wr, xv, wt4, xrow, Epad, col, wave, lane, 0);
+    rl_stash(lds, wr, xv, wave, lane);
+    rl_fetch(wr, xv, wt4, xrow, Epad, col, wave, lane, min(1, nchunk - 1));
+    for (int c = 0; c < nchunk; ++c) {
+        __syncthreads();   // slot c % 2 is complete; nobody reads slot (c + 1) % 2 any more
+        // past the last chunk both lines repeat it into the slot nobody reads any more: no branch around loads
+        rl_stash(lds + ((c + 1) & 1) * (RL_W_SLOT + RL_X_SLOT), wr, xv, wave, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        rl_fetch(wr, xv, wt4, xrow, Epad, col, wave, lane, min(c + 2, nchunk - 1));
+        __builtin_amdgcn_sched_barrier(0);
+        const rl_f4* w = lds + (c & 1) * (RL_W_SLOT + RL_X_SLOT);
+        const rl_f4* xs = w + RL_W_SLOT + wave * (RL_KC / 4);
+#pragma unroll 8
+        for (int q = 0; q < RL_KC / 4; ++q) {
+            const rl_f4 wq = w[q * 64 + lane], xq = xs[q];
+            acc = fadd(acc, fmul(xq[0], wq[0]));
+            acc = fadd(acc, fmul(xq[1], wq[1]));
+            acc = fadd(acc, fmul(xq[2], wq[2]));
+            acc = fadd(acc, fmul(xq[3], wq[3]));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (t < n && col < E) logits[(size_t)t * E + col] = acc;
+}
+
 template <typename XT, int T>
 static int launch_router_tile_t(const XT* xp, const float4* wp, int n, int H, int E, int Epad, float* logits,
                                 hipStream_t st) {
@@ -1151,18 +1235,26 @@ static int launch_router_tile_t(const XT* xp, const float4* wp, int n, int H, in
     return check_launch("router_tile");
 }
 
-// Tokens per wave: four share a wave's weight loads, but a wave walks its chains one after the other, so with few
-// tokens the kernel's time is the length of one wave's work (320 tokens x 128 experts at four tokens per wave are
-// 160 waves on 1024 SIMDs: 114 us).  Fewer tokens per wave while that leaves SIMDs idle.
+// Four tokens per wave in registers for thousands of tokens, two for a thousand or two (more waves), and the
+// LDS-sharing kernel below that.
 template <typename XT>
 static int launch_router_tile(const void* x, const float* router_t, int n, int H, int E, float* logits, hipStream_t st) {
     const int Epad = (E + 63) / 64 * 64;
     const XT* xp = static_cast<const XT*>(x);
     const float4* wp = reinterpret_cast<const float4*>(router_t);
     const long groups = Epad / 64;
-    if (groups * ((n + 3) / 4) >= 1024) return launch_router_tile_t<XT, 4>(xp, wp, n, H, E, Epad, logits, st);
-    if (groups * ((n + 1) / 2) >= 1024) return launch_router_tile_t<XT, 2>(xp, wp, n, H, E, Epad, logits, st);
-    return launch_router_tile_t<XT, 1>(xp, wp, n, H, E, Epad, logits, st);
+    // measured at 128 experts, H 4096: 320 / 512 / 767 / 1024 tokens 48 / 49 / 61 / 63 us with the LDS-sharing kernel
+    // (79 / 80 / 85 / 86 us with one token per wave of the register-tiled kernel, 115 us with four); 1536 / 2048
+    // tokens 97 / 98 us with two tokens per wave (101 / 117 us LDS-sharing, 115 / 116 us with four)
+    if (groups * n <= 2048) {
+        int rc = LdsLimit<&router_lds_kernel<XT>>::ensure(RL_LDS_BYTES);
+        if (rc) return rc;
+        dim3 grid((unsigned)groups, (n + 3) / 4);
+        router_lds_kernel<XT><<<grid, 256, RL_LDS_BYTES, st>>>(xp, wp, n, H, E, Epad, logits);
+        return check_launch("router_lds");
+    }
+    if (groups * n <= 4096) return launch_router_tile_t<XT, 2>(xp, wp, n, H, E, Epad, logits, st);
+    return launch_router_tile_t<XT, 4>(xp, wp, n, H, E, Epad, logits, st);
 }
 
 // Router GEMM alone from the transposed weight (any n): logits only.

@@ -508,16 +508,19 @@ def test_layer_all_tokens_on_the_same_experts(hip, oracle, n):
         check_mfma(hip, oracle, layer, inp, MODE_MFMA_FP8_X2, ref32)
 
 
-@pytest.mark.parametrize("n,experts", [(300, 128), (600, 256), (1100, 256), (2100, 512)])
-def test_router_chain_tokens_per_wave(hip, oracle, n, experts):
-    """Beyond 256 tokens the router chain runs register-tiled, one, two or four tokens per wave by how many waves
-    that leaves (300 x 128: one; 600 x 256: two; 1100 x 256 and 2100 x 512: four, the last with two expert blocks per
-    wave): the same sequential-k f32 chain in every form, so logits, ids, probabilities and the permutation tables
-    are the oracle's bit for bit."""
-    cfg = synth.MoeConfig(n, 256, experts, 4, 128, 128, 8, 4)
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("n,experts,hidden", [(300, 128, 256), (1000, 64, 384), (600, 256, 256), (1100, 256, 256),
+                                              (2100, 512, 256)])
+def test_router_chain_forms(hip, oracle, n, experts, hidden, bf16):
+    """Beyond 256 tokens the router chain has three forms, chosen by tokens x expert blocks: four waves that share a
+    chunk of the weights through LDS, one token each (300 x 128, 1000 x 64); register-tiled with two tokens per wave
+    (600 x 256) or four (1100 x 256; 2100 x 512 with two expert blocks per wave).  All walk the same sequential-k f32
+    chain, so logits, ids, probabilities and the permutation tables are the oracle's bit for bit, for f32 and bf16
+    activations."""
+    cfg = synth.MoeConfig(n, hidden, experts, 4, 128, 128, 8, 4, act_bf16=bf16)
     inp = synth.make_inputs(cfg, seed=n)
     layer = hip.load_moe_layer(inp, keep_checkpoint_layout=False)
-    _, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8)
+    _, v = run_layer(hip, layer, inp.x, MODE_MFMA_FP8, bf16=bf16)
     check_routing(v, oracle.moe_ffn_mxfp4(inp, n_threads=8, want_out=False), oracle, cfg)
 
 
