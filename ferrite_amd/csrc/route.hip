@@ -1017,7 +1017,7 @@ static int warmup_head() {
     return LdsLimit<&moe_head_kernel<XT, kFused, 2, 32>>::ensure(cap);
 }
 
-template <typename XT> __global__ void router_lds_kernel(const XT*, const float4*, int, int, int, int, float*);
+template <typename XT> __global__ __launch_bounds__(256) void router_lds_kernel(const XT*, const float4*, int, int, int, int, float*);
 
 int warmup_route() {
     int rc;
@@ -1189,9 +1189,12 @@ __global__ __launch_bounds__(256) void router_lds_kernel(const XT* __restrict__ 
     const int col = blockIdx.x * 64 + lane;
     const XT* xrow = x + (size_t)min(t, n - 1) * H;
     const int nchunk = H / RL_KC;
-    // One register set: chunk c + 1 is in flight while chunk c is walked.  (Two sets, a chunk fetched two chunk
-    // times ahead, measured slower: 67 against 48 us at 320 tokens.  What bounds a block is LDS bandwidth - 160 KiB
-    // of reads and writes per chunk - and the chains' own instructions, one after the other in a lone wave.)
+    // One register set: chunk c + 1 is in flight while chunk c is walked.  What bounds a block is LDS bandwidth:
+    // four waves read 1 KiB of weights each per four k, eight cycles per k, and with the chains' own instructions
+    // on top a block takes 46-48 us at H 4096 (31 us with the multiplies compiled out).  Measured and not kept: a
+    // second register set, a chunk fetched two chunk times ahead (67 us); the next group's LDS reads issued before
+    // the current group's chain (46 us); the activations taken with v_readlane from registers instead of broadcast
+    // LDS reads (50 us).
     rl_f4 wr[RL_KC / 16];
     float xv[2];
     float acc = 0.0f;
